@@ -1,0 +1,95 @@
+"""ctypes binding of libmegagemm_hip.so (the C ABI declared in include/megagemm_hip.h).
+
+This is the only module that touches the shared library.  It takes the place of the
+reference's pybind11 extension module `rmsnorm_cuda_ops` (pytorch_binding/binding.cpp)
+and of the Triton launch sites in megagemm/swiglu.py:100-107,122-129.
+
+There is no CPU fallback: if the library is missing or a call fails, a RuntimeError is
+raised with the library's own message.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "libmegagemm_hip.so"
+ABI_VERSION = 1
+
+MG_F32, MG_F16, MG_BF16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: MG_F32, torch.float16: MG_F16, torch.bfloat16: MG_BF16}
+
+_lock = threading.Lock()
+_lib = None
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+# name -> (restype, argtypes); mirrors include/megagemm_hip.h one to one
+SIGNATURES = {
+    "mg_abi_version": (_int, []),
+    "mg_last_error": (ctypes.c_char_p, []),
+    "mg_set_option": (_int, [ctypes.c_char_p, _int]),
+    "mg_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _int, _vp]),
+    "mg_rmsnorm_bwd_workspace": (_int, [_i64, _i64, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64)]),
+    "mg_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _i64, _vp]),
+    "mg_rmsnorm_dw_reduce": (_int, [_vp, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
+    "mg_swiglu_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
+    "mg_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
+}
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once per process; raise RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"HIP library not built: {LIB_PATH} is missing. "
+                "Run: python -m mgrrmsnorm_amd._build   (needs hipcc; builds for gfx950)")
+        try:
+            lib = ctypes.CDLL(str(LIB_PATH))
+        except OSError as exc:  # e.g. libamdhip64.so not found
+            raise RuntimeError(f"cannot load {LIB_PATH}: {exc}") from exc
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = lib.mg_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} has ABI version {got}, this package needs {ABI_VERSION}; rebuild it")
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().mg_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed (code {rc}): {last_error()}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError(
+            f"Unsupported dtype {dtype}. Use float32, float16, or bfloat16.") from None
+
+
+def stream_ptr(device: torch.device) -> int:
+    """Raw hipStream_t of torch's current stream on `device`."""
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def set_option(key: str, value: int) -> None:
+    check(load().mg_set_option(key.encode(), int(value)), "mg_set_option")

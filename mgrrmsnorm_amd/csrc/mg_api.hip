@@ -1,0 +1,333 @@
+// C ABI of libmegagemm_hip.so: argument validation, choice of launch shape, launch.
+// Validation happens before any HIP call so that argument errors are reported on hosts
+// without a GPU.
+#include "megagemm_hip.h"
+#include "mg_launch.hpp"
+#include "mg_device.hpp"
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+namespace mg {
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int fail_hip(const char* what, hipError_t e) {
+    return fail(MG_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+// ---- process-wide tuning overrides (0 / -1 = automatic) ----
+std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_items{0}, opt_bwd_wg_per_cu{0},
+    opt_swiglu_unroll{0}, opt_force_generic{0};
+
+int esize_of(int dtype) {
+    switch (dtype) {
+        case MG_F32: return 4;
+        case MG_F16: return 2;
+        case MG_BF16: return 2;
+        default: return 0;
+    }
+}
+
+const char* dtype_name(int dtype) {
+    switch (dtype) {
+        case MG_F32: return "fp32";
+        case MG_F16: return "fp16";
+        case MG_BF16: return "bf16";
+        default: return "?";
+    }
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+// Compute units of the current device (cached per device ordinal).
+int cu_count(int* out) {
+    static std::atomic<int> cache[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail_hip("hipGetDevice", e);
+    if (dev >= 0 && dev < 64) {
+        int c = cache[dev].load(std::memory_order_relaxed);
+        if (c > 0) { *out = c; return MG_OK; }
+    }
+    int n = 0;
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return fail_hip("hipDeviceGetAttribute(MultiprocessorCount)", e);
+    if (n <= 0) n = 256;
+    if (dev >= 0 && dev < 64) cache[dev].store(n, std::memory_order_relaxed);
+    *out = n;
+    return MG_OK;
+}
+
+int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
+
+// Vector width the register-resident kernels can use for this row pitch and these bases:
+// 16, 8, or 0 (generic kernels).
+int pick_vec(long row_bytes, std::initializer_list<const void*> ptrs) {
+    int v = (row_bytes % 16 == 0) ? 16 : (row_bytes % 8 == 0) ? 8 : 0;
+    if (v == 0) return 0;
+    for (const void* p : ptrs)
+        if (p != nullptr && !aligned(p, 16)) return 0;
+    return v;
+}
+
+int round_items_fwd(int items) { return items == 7 ? 8 : items; }
+
+// Forward: the fewest threads per row that keep a thread at or below `target` vectors.
+bool choose_fwd(long row_bytes, int vec, RowCfg* cfg) {
+    const long nvec = row_bytes / vec;
+    int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
+    if (tpr_ok(tpr)) {
+        const int need = round_items_fwd(ceil_div(nvec, tpr));
+        if (need <= kFwdMaxItems && fwd_items_ok(need)) { *cfg = {vec, tpr, need}; return true; }
+    }
+    const int target = (items > 0 && items <= kFwdMaxItems) ? items : 2;
+    for (int t = 64; t <= 1024; t *= 2) {
+        const int need = round_items_fwd(ceil_div(nvec, t));
+        if (need <= target || (t == 1024 && need <= kFwdMaxItems)) { *cfg = {vec, t, need}; return true; }
+    }
+    return false;
+}
+
+bool choose_bwd(long row_bytes, int esize, int vec, RowCfg* cfg) {
+    const long nvec = row_bytes / vec;
+    int tpr = opt_bwd_tpr.load(), items = opt_bwd_items.load();
+    if (tpr_ok(tpr)) {
+        const int need = ceil_div(nvec, tpr);
+        if (bwd_cfg_ok(esize, vec, tpr, need)) { *cfg = {vec, tpr, need}; return true; }
+    }
+    const int target = (items > 0 && items <= kBwdMaxItems) ? items : 2;
+    for (int t = 64; t <= 1024; t *= 2) {
+        const int need = ceil_div(nvec, t);
+        if ((need <= target || t == 1024) && bwd_cfg_ok(esize, vec, t, need)) { *cfg = {vec, t, need}; return true; }
+    }
+    return false;
+}
+
+int check_rmsnorm_dims(const char* fn, int64_t rows, int64_t cols, int dtype) {
+    const int es = esize_of(dtype);
+    if (es == 0) return fail(MG_ERR_INVALID_ARG, "%s: unknown dtype %d (use 0=fp32, 1=fp16, 2=bf16)", fn, dtype);
+    if (rows < 0) return fail(MG_ERR_INVALID_ARG, "%s: rows must be >= 0 (got %lld)", fn, (long long)rows);
+    if (cols < 1) return fail(MG_ERR_INVALID_ARG, "%s: cols must be >= 1 (got %lld)", fn, (long long)cols);
+    if (cols * es >= (1LL << 31))
+        return fail(MG_ERR_UNSUPPORTED, "%s: cols too large (%lld %s elements; a row must stay below 2 GiB)", fn,
+                    (long long)cols, dtype_name(dtype));
+    if (rows >= (1LL << 31))
+        return fail(MG_ERR_UNSUPPORTED, "%s: rows too large (%lld; max 2^31-1)", fn, (long long)rows);
+    return MG_OK;
+}
+
+template <typename F32, typename F16, typename BF16>
+hipError_t by_dtype(int dtype, F32 f32, F16 f16, BF16 bf16) {
+    switch (dtype) {
+        case MG_F32: return f32();
+        case MG_F16: return f16();
+        default: return bf16();
+    }
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_abi_version(void) { return MG_ABI_VERSION; }
+
+const char* mg_last_error(void) { return g_err; }
+
+int mg_set_option(const char* key, int value) {
+    if (key == nullptr) return fail(MG_ERR_INVALID_ARG, "mg_set_option: key is NULL");
+    struct { const char* k; std::atomic<int>* v; } table[] = {
+        {"fwd_tpr", &opt_fwd_tpr},       {"fwd_items", &opt_fwd_items},
+        {"bwd_tpr", &opt_bwd_tpr},       {"bwd_items", &opt_bwd_items},
+        {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
+        {"force_generic", &opt_force_generic},
+    };
+    for (auto& t : table)
+        if (strcmp(t.k, key) == 0) { t.v->store(value); return MG_OK; }
+    return fail(MG_ERR_INVALID_ARG, "mg_set_option: unknown key '%s'", key);
+}
+
+int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_t rows, int64_t cols, float eps,
+                   int dtype, void* stream) {
+    int rc = check_rmsnorm_dims("mg_rmsnorm_fwd", rows, cols, dtype);
+    if (rc != MG_OK) return rc;
+    if (rows == 0) return MG_OK;
+    if (y == nullptr || x == nullptr || w == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_fwd: y, x and w must not be NULL");
+    const int es = esize_of(dtype);
+    if (!aligned(y, es) || !aligned(x, es) || !aligned(w, es) || !aligned(inv_rms, 4))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_fwd: a pointer is not aligned to its element size");
+
+    const long row_bytes = cols * es;
+    RowCfg cfg = {0, 0, 0};
+    bool generic = opt_force_generic.load() != 0;
+    if (!generic) {
+        const int vec = pick_vec(row_bytes, {y, x, w});
+        generic = (vec == 0) || !choose_fwd(row_bytes, vec, &cfg);
+    }
+    const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps};
+    hipStream_t s = (hipStream_t)stream;
+    hipError_t e = by_dtype(
+        dtype, [&] { return launch_rmsnorm_fwd<float>(cfg, generic, a, s); },
+        [&] { return launch_rmsnorm_fwd<half_t>(cfg, generic, a, s); },
+        [&] { return launch_rmsnorm_fwd<bf16_t>(cfg, generic, a, s); });
+    if (e != hipSuccess) return fail_hip("mg_rmsnorm_fwd: launch", e);
+    return MG_OK;
+}
+
+int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num_partials, int64_t* ld) {
+    int rc = check_rmsnorm_dims("mg_rmsnorm_bwd_workspace", rows, cols, dtype);
+    if (rc != MG_OK) return rc;
+    if (num_partials == nullptr || ld == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd_workspace: output pointers must not be NULL");
+    *ld = (cols + 63) / 64 * 64;
+    if (rows == 0) { *num_partials = 1; return MG_OK; }
+    int cus = 0;
+    rc = cu_count(&cus);
+    if (rc != MG_OK) return rc;
+    int per_cu = opt_bwd_wg_per_cu.load();
+    if (per_cu < 1 || per_cu > 8) per_cu = 1;
+    // one persistent workgroup per compute unit; fewer when there are not enough rows
+    // to give every row slot of every workgroup at least one row
+    const int es = esize_of(dtype);
+    RowCfg cfg = {0, 0, 0};
+    const int vec = (cols * es % 16 == 0) ? 16 : (cols * es % 8 == 0) ? 8 : 0;
+    int rg = 1;
+    if (vec != 0 && opt_force_generic.load() == 0 && choose_bwd(cols * es, es, vec, &cfg)) rg = 1024 / cfg.tpr;
+    int64_t p = (int64_t)cus * per_cu;
+    const int64_t by_rows = (rows + rg - 1) / rg;
+    if (p > by_rows) p = by_rows;
+    if (p < 1) p = 1;
+    if (p > 65535) p = 65535;
+    *num_partials = p;
+    return MG_OK;
+}
+
+int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, const void* w, const float* inv_rms,
+                   int64_t rows, int64_t cols, int dtype, int64_t num_partials, int64_t ld, void* stream) {
+    int rc = check_rmsnorm_dims("mg_rmsnorm_bwd", rows, cols, dtype);
+    if (rc != MG_OK) return rc;
+    if (num_partials < 1 || num_partials > 65535)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: num_partials must be in [1, 65535] (got %lld)",
+                    (long long)num_partials);
+    if (ld < cols || ld % 64 != 0 || ld >= (1LL << 31))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: ld must be a multiple of 64 and >= cols (got %lld)",
+                    (long long)ld);
+    if (dw_partial == nullptr || !aligned(dw_partial, 16))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: dw_partial must be a 16-byte aligned device pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (rows == 0) {
+        hipError_t e = launch_fill_zero(dw_partial, (long)(num_partials * ld), s);
+        if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd: zero fill", e);
+        return MG_OK;
+    }
+    if (dx == nullptr || dy == nullptr || x == nullptr || w == nullptr || inv_rms == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: dx, dy, x, w and inv_rms must not be NULL");
+    const int es = esize_of(dtype);
+    if (!aligned(dx, es) || !aligned(dy, es) || !aligned(x, es) || !aligned(w, es) || !aligned(inv_rms, 4))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: a pointer is not aligned to its element size");
+
+    const long row_bytes = cols * es;
+    RowCfg cfg = {0, 0, 0};
+    bool generic = opt_force_generic.load() != 0;
+    if (!generic) {
+        const int vec = pick_vec(row_bytes, {dx, dy, x, w});
+        generic = (vec == 0) || !choose_bwd(row_bytes, es, vec, &cfg);
+    }
+    const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials};
+    hipError_t e = by_dtype(
+        dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },
+        [&] { return launch_rmsnorm_bwd<half_t>(cfg, generic, a, s); },
+        [&] { return launch_rmsnorm_bwd<bf16_t>(cfg, generic, a, s); });
+    if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd: launch", e);
+    return MG_OK;
+}
+
+int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* dw_partial,
+                         int64_t num_partials, int64_t ld, int64_t cols, void* stream) {
+    if (cols < 1 || cols >= (1LL << 31))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: cols must be in [1, 2^31) (got %lld)", (long long)cols);
+    if (num_partials < 1 || num_partials > 65535)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: num_partials must be in [1, 65535] (got %lld)",
+                    (long long)num_partials);
+    if (ld < cols || ld % 64 != 0 || ld >= (1LL << 31))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: ld must be a multiple of 64 and >= cols (got %lld)",
+                    (long long)ld);
+    if (dw_f32 == nullptr && dw_cast == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: give dw_f32, dw_cast or both");
+    if (dw_cast != nullptr && esize_of(cast_dtype) == 0)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: unknown cast_dtype %d", cast_dtype);
+    if (dw_partial == nullptr || !aligned(dw_partial, 16))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: dw_partial must be a 16-byte aligned device pointer");
+    if (!aligned(dw_f32, 4) || (dw_cast != nullptr && !aligned(dw_cast, esize_of(cast_dtype))))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: an output pointer is not aligned to its element size");
+    hipError_t e = launch_dw_reduce(dw_f32, dw_cast, cast_dtype, dw_partial, (int)num_partials, (int)ld, (int)cols,
+                                    (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip("mg_rmsnorm_dw_reduce: launch", e);
+    return MG_OK;
+}
+
+static int check_swiglu(const char* fn, int64_t M, int64_t H, int dtype) {
+    if (esize_of(dtype) == 0)
+        return fail(MG_ERR_INVALID_ARG, "%s: unknown dtype %d (use 0=fp32, 1=fp16, 2=bf16)", fn, dtype);
+    if (M < 0) return fail(MG_ERR_INVALID_ARG, "%s: M must be >= 0 (got %lld)", fn, (long long)M);
+    if (H < 1) return fail(MG_ERR_INVALID_ARG, "%s: H must be >= 1 (got %lld)", fn, (long long)H);
+    if (H >= (1LL << 30)) return fail(MG_ERR_UNSUPPORTED, "%s: H too large (%lld; max 2^30-1)", fn, (long long)H);
+    if (M > (1LL << 40) / H)
+        return fail(MG_ERR_UNSUPPORTED, "%s: M*H too large (%lld x %lld; max 2^40 elements)", fn, (long long)M,
+                    (long long)H);
+    return MG_OK;
+}
+
+static int swiglu_unroll(int dflt, int maxv) {
+    int u = opt_swiglu_unroll.load();
+    if (u == 1 || u == 2 || u == 4 || (u == 8 && maxv >= 8)) return u;
+    return dflt;
+}
+
+int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void* stream) {
+    int rc = check_swiglu("mg_swiglu_fwd", M, H, dtype);
+    if (rc != MG_OK) return rc;
+    if (M == 0) return MG_OK;
+    if (h == nullptr || gu == nullptr) return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: h and gu must not be NULL");
+    const int es = esize_of(dtype);
+    if (!aligned(h, es) || !aligned(gu, es))
+        return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: a pointer is not aligned to its element size");
+    const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(h, 16) && aligned(gu, 16);
+    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(4, 8), h, gu, (long)M, (long)H, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip("mg_swiglu_fwd: launch", e);
+    return MG_OK;
+}
+
+int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t H, int dtype, void* stream) {
+    int rc = check_swiglu("mg_swiglu_bwd", M, H, dtype);
+    if (rc != MG_OK) return rc;
+    if (M == 0) return MG_OK;
+    if (dgu == nullptr || dh == nullptr || gu == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_swiglu_bwd: dgu, dh and gu must not be NULL");
+    const int es = esize_of(dtype);
+    if (!aligned(dgu, es) || !aligned(dh, es) || !aligned(gu, es))
+        return fail(MG_ERR_INVALID_ARG, "mg_swiglu_bwd: a pointer is not aligned to its element size");
+    const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(dgu, 16) && aligned(dh, 16) &&
+                     aligned(gu, 16);
+    hipError_t e =
+        launch_swiglu_bwd(dtype, vec, swiglu_unroll(2, 4), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip("mg_swiglu_bwd: launch", e);
+    return MG_OK;
+}
+
+}  // extern "C"

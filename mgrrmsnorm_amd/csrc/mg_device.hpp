@@ -1,0 +1,154 @@
+// Device-side building blocks shared by the gfx950 kernels: 128/64-bit raw buffer
+// loads and stores, element packing for fp32/fp16/bf16, wave64 DPP reduction.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mg {
+
+typedef unsigned int u32;
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+typedef _Float16 half_t;
+typedef __bf16 bf16_t;
+
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------------
+// Raw buffer resources.  A resource describes [base, base + bytes): loads whose byte
+// offset falls outside return 0 and stores outside are dropped, which gives branch-free
+// row tails and lets a wave that has no row left run with bytes == 0.
+// Word 3 = 0x00020000 selects the untyped 32-bit data format on gfx9-family parts.
+// ---------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, u32 bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// NW 32-bit words per vector (4 -> dwordx4, 2 -> dwordx2).
+template <int NW> struct Words { u32 v[NW]; };
+
+template <int NW>
+__device__ __forceinline__ Words<NW> buf_load(rsrc_t r, u32 byte_off);
+template <>
+__device__ __forceinline__ Words<4> buf_load<4>(rsrc_t r, u32 byte_off) {
+    u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
+    Words<4> o; o.v[0] = t.x; o.v[1] = t.y; o.v[2] = t.z; o.v[3] = t.w; return o;
+}
+template <>
+__device__ __forceinline__ Words<2> buf_load<2>(rsrc_t r, u32 byte_off) {
+    u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0);
+    Words<2> o; o.v[0] = t.x; o.v[1] = t.y; return o;
+}
+
+template <int NW>
+__device__ __forceinline__ void buf_store(rsrc_t r, u32 byte_off, const Words<NW>& w);
+template <>
+__device__ __forceinline__ void buf_store<4>(rsrc_t r, u32 byte_off, const Words<4>& w) {
+    u32x4 t = {w.v[0], w.v[1], w.v[2], w.v[3]};
+    __builtin_amdgcn_raw_buffer_store_b128(t, r, (int)byte_off, 0, 0);
+}
+template <>
+__device__ __forceinline__ void buf_store<2>(rsrc_t r, u32 byte_off, const Words<2>& w) {
+    u32x2 t = {w.v[0], w.v[1]};
+    __builtin_amdgcn_raw_buffer_store_b64(t, r, (int)byte_off, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------
+// Element traits: PER_WORD elements per 32-bit word, conversion to/from fp32.
+// fp32 -> fp16/bf16 uses the hardware round-to-nearest-even converts
+// (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32); never the round-toward-zero pack.
+// ---------------------------------------------------------------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<float> {
+    static constexpr int PER_WORD = 1;
+    static __device__ __forceinline__ void unpack(u32 w, float* f) { f[0] = __builtin_bit_cast(float, w); }
+    static __device__ __forceinline__ u32 pack(const float* f) { return __builtin_bit_cast(u32, f[0]); }
+    static __device__ __forceinline__ float load1(const float* p) { return *p; }
+    static __device__ __forceinline__ void store1(float* p, float f) { *p = f; }
+};
+
+template <> struct Elem<half_t> {
+    static constexpr int PER_WORD = 2;
+    static __device__ __forceinline__ void unpack(u32 w, float* f) {
+        f16x2 h = __builtin_bit_cast(f16x2, w);
+        f[0] = (float)h.x; f[1] = (float)h.y;
+    }
+    static __device__ __forceinline__ u32 pack(const float* f) {
+        f32x2 p = {f[0], f[1]};
+        return __builtin_bit_cast(u32, __builtin_convertvector(p, f16x2));
+    }
+    static __device__ __forceinline__ float load1(const half_t* p) { return (float)*p; }
+    static __device__ __forceinline__ void store1(half_t* p, float f) { *p = (half_t)f; }
+};
+
+template <> struct Elem<bf16_t> {
+    static constexpr int PER_WORD = 2;
+    static __device__ __forceinline__ void unpack(u32 w, float* f) {
+        f[0] = __builtin_bit_cast(float, w << 16);
+        f[1] = __builtin_bit_cast(float, w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ u32 pack(const float* f) {
+        f32x2 p = {f[0], f[1]};
+        return __builtin_bit_cast(u32, __builtin_convertvector(p, bf16x2));
+    }
+    static __device__ __forceinline__ float load1(const bf16_t* p) {
+        unsigned short b = *reinterpret_cast<const unsigned short*>(p);
+        return __builtin_bit_cast(float, (u32)b << 16);
+    }
+    static __device__ __forceinline__ void store1(bf16_t* p, float f) { *p = (bf16_t)f; }
+};
+
+// Unpack / pack a whole vector of NW words = NW * PER_WORD elements.
+template <typename T, int NW>
+__device__ __forceinline__ void unpack_vec(const Words<NW>& w, float* f) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) Elem<T>::unpack(w.v[i], f + i * Elem<T>::PER_WORD);
+}
+template <typename T, int NW>
+__device__ __forceinline__ Words<NW> pack_vec(const float* f) {
+    Words<NW> w;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) w.v[i] = Elem<T>::pack(f + i * Elem<T>::PER_WORD);
+    return w;
+}
+
+// ---------------------------------------------------------------------------------
+// wave64 all-reduce (sum).  Four DPP steps make every lane of each 16-lane row hold that
+// row's sum (xor-1, xor-2 inside quads, then rotate-by-4 and rotate-by-8 inside the row);
+// the four row sums are then read with v_readlane and added in a fixed order, so the
+// result is identical in all 64 lanes and from run to run.
+// ---------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_mov<0x124>(v);  // row_ror:4
+    v += dpp_mov<0x128>(v);  // row_ror:8
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
+
+__device__ __forceinline__ float fast_rsqrt(float v) { return __builtin_amdgcn_rsqf(v); }
+
+// sigmoid(g) = 1 / (1 + 2^(-g*log2(e))).  For g << 0 the power overflows to +inf and the
+// reciprocal gives +0, the correct limit.
+__device__ __forceinline__ float fast_sigmoid(float g) {
+    float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+    return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+}  // namespace mg

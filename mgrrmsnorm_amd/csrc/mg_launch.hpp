@@ -1,0 +1,54 @@
+// Internal interface between the C ABI (mg_api.hip) and the per-dtype kernel
+// translation units.  Everything here is host code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mg {
+
+// How a row is spread over threads in the register-resident RMSNorm kernels.
+struct RowCfg {
+    int vec;    // bytes per vector load: 16 or 8
+    int tpr;    // threads per row: 64, 128, 256, 512, 1024
+    int items;  // vectors per thread
+};
+
+// Largest ITEMS instantiated.
+constexpr int kFwdMaxItems = 8;
+constexpr int kBwdMaxItems = 4;
+
+// Forward: ITEMS in {1,2,3,4,5,6,8}.
+constexpr bool fwd_items_ok(int items) { return items >= 1 && items <= 8 && items != 7; }
+// Backward: ITEMS in {1,2,3,4}; when several row slots share a workgroup their combine
+// buffer (tpr * items * elements-per-vector floats) must fit 64 KiB of LDS.
+constexpr bool bwd_cfg_ok(int esize, int vec, int tpr, int items) {
+    return items >= 1 && items <= kBwdMaxItems &&
+           (tpr == 1024 || tpr * items * (vec / esize) * 4 <= 65536);
+}
+constexpr bool tpr_ok(int tpr) { return tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024; }
+
+struct FwdArgs {
+    void* y; float* inv_rms; const void* x; const void* w;
+    long rows; int cols; float eps;
+};
+struct BwdArgs {
+    void* dx; float* dw_part; int ld; const void* dy; const void* x; const void* w; const float* inv_rms;
+    long rows; int cols; int num_partials;
+};
+
+// One set of launchers per element type (T = float, _Float16, __bf16), each defined in
+// its own translation unit.  `generic` selects the element-wise kernels.
+template <typename T> hipError_t launch_rmsnorm_fwd(const RowCfg& cfg, bool generic, const FwdArgs& a, hipStream_t s);
+template <typename T> hipError_t launch_rmsnorm_bwd(const RowCfg& cfg, bool generic, const BwdArgs& a, hipStream_t s);
+
+hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* part, int P, int ld,
+                            int cols, hipStream_t s);
+hipError_t launch_fill_zero(float* p, long n, hipStream_t s);
+
+// SwiGLU: `vec` = true takes the 16-byte kernels (requires H*sizeof(T) % 16 == 0 and
+// 16-byte aligned bases).  rows*H per launch must stay below 2^31 units (vectors or elements).
+hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H, hipStream_t s);
+hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M,
+                             long H, hipStream_t s);
+
+}  // namespace mg

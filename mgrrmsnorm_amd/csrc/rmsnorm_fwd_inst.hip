@@ -1,0 +1,73 @@
+// RMSNorm forward launchers for one element type; compile with -DMG_DTYPE=0|1|2
+// (fp32 | fp16 | bf16).
+#include "mg_launch.hpp"
+#include "rmsnorm_kernels.hpp"
+
+#ifndef MG_DTYPE
+#error "compile with -DMG_DTYPE=0 (fp32), 1 (fp16) or 2 (bf16)"
+#endif
+
+namespace mg {
+namespace {
+
+#if MG_DTYPE == 0
+typedef float elem_t;
+#elif MG_DTYPE == 1
+typedef half_t elem_t;
+#else
+typedef bf16_t elem_t;
+#endif
+
+template <int VEC, int TPR, int ITEMS>
+hipError_t run(const FwdArgs& a, hipStream_t s) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    const long grid = (a.rows + RPB - 1) / RPB;
+    rmsnorm_fwd_rows<elem_t, VEC, TPR, ITEMS><<<dim3((unsigned)grid), dim3(BLOCK), 0, s>>>(
+        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+        1.0f / (float)a.cols);
+    return hipGetLastError();
+}
+
+template <int VEC, int TPR>
+hipError_t by_items(int items, const FwdArgs& a, hipStream_t s) {
+    switch (items) {
+        case 1: return run<VEC, TPR, 1>(a, s);
+        case 2: return run<VEC, TPR, 2>(a, s);
+        case 3: return run<VEC, TPR, 3>(a, s);
+        case 4: return run<VEC, TPR, 4>(a, s);
+        case 5: return run<VEC, TPR, 5>(a, s);
+        case 6: return run<VEC, TPR, 6>(a, s);
+        case 8: return run<VEC, TPR, 8>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <int VEC>
+hipError_t by_tpr(int tpr, int items, const FwdArgs& a, hipStream_t s) {
+    switch (tpr) {
+        case 64: return by_items<VEC, 64>(items, a, s);
+        case 128: return by_items<VEC, 128>(items, a, s);
+        case 256: return by_items<VEC, 256>(items, a, s);
+        case 512: return by_items<VEC, 512>(items, a, s);
+        case 1024: return by_items<VEC, 1024>(items, a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+template <>
+hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const FwdArgs& a, hipStream_t s) {
+    if (generic) {
+        rmsnorm_fwd_generic<elem_t><<<dim3((unsigned)a.rows), dim3(256), 0, s>>>(
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+            1.0f / (float)a.cols);
+        return hipGetLastError();
+    }
+    if (cfg.vec == 16) return by_tpr<16>(cfg.tpr, cfg.items, a, s);
+    if (cfg.vec == 8) return by_tpr<8>(cfg.tpr, cfg.items, a, s);
+    return hipErrorInvalidValue;
+}
+
+}  // namespace mg

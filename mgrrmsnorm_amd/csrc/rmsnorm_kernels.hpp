@@ -1,0 +1,361 @@
+// RMSNorm forward / backward kernels for gfx950.
+//
+// Register-resident family ("rows" kernels): a row of `cols` elements is split into
+// vectors of VEC bytes; TPR threads (a multiple of the 64-lane wave) share one row and
+// each holds ITEMS vectors of it in VGPRs, vector i of thread t being vector t + i*TPR of
+// the row.  All of a row's loads are issued before the first use.  Row sums are reduced
+// with DPP inside a wave and through a few floats of LDS across the waves of a row.
+//
+// Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
+// the row; used when the row pitch is not a multiple of 8 bytes, a base pointer is not
+// 16-byte aligned, or the row does not fit the register-resident family.
+#pragma once
+#include "mg_device.hpp"
+
+namespace mg {
+
+// =================================================================================
+// Forward, register-resident.
+//   grid  = ceil(rows / RPB) workgroups, RPB = BLOCK / TPR rows per workgroup
+//   block = BLOCK = max(TPR, 256) threads
+// =================================================================================
+template <typename T, int VEC, int TPR, int ITEMS>
+__global__ void __launch_bounds__((TPR > 256 ? TPR : 256))
+rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                 const T* __restrict__ w, long rows, int cols, float eps, float inv_cols) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    constexpr int WPR = TPR / kWave;
+    constexpr int NW = VEC / 4;
+    constexpr int EPV = VEC / (int)sizeof(T);
+
+    const int tid = threadIdx.x;
+    const int rg = __builtin_amdgcn_readfirstlane(tid / TPR);  // row slot inside the workgroup
+    const int lir = tid - rg * TPR;                            // lane inside the row
+    const long row = (long)blockIdx.x * RPB + rg;
+    const bool live = row < rows;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const long base = live ? row * (long)cols : 0;
+
+    const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
+    const rsrc_t ry = make_rsrc(y + base, live ? row_bytes : 0u);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+
+    Words<NW> xv[ITEMS];
+    Words<NW> wv[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW>(rw, (u32)(lir + i * TPR) * VEC);
+
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float f[EPV];
+        unpack_vec<T, NW>(xv[i], f);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) ss = __builtin_fmaf(f[k], f[k], ss);
+    }
+    ss = wave_sum(ss);
+    if constexpr (WPR > 1) {
+        __shared__ float part[RPB][WPR];
+        const int wir = __builtin_amdgcn_readfirstlane(lir / kWave);  // wave inside the row
+        if ((tid & (kWave - 1)) == 0) part[rg][wir] = ss;
+        __syncthreads();
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < WPR; ++k) t += part[rg][k];
+        ss = t;
+    }
+    const float s = fast_rsqrt(ss * inv_cols + eps);
+    if (live && lir == 0 && inv_rms != nullptr) inv_rms[row] = s;
+
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float xf[EPV], wf[EPV], o[EPV];
+        unpack_vec<T, NW>(xv[i], xf);
+        unpack_vec<T, NW>(wv[i], wf);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
+        buf_store<NW>(ry, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+    }
+}
+
+// =================================================================================
+// Forward, generic: one workgroup of 256 threads per row, any cols, any alignment.
+// =================================================================================
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_fwd_generic(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                    const T* __restrict__ w, long rows, int cols, float eps, float inv_cols) {
+    const long row = blockIdx.x;
+    if (row >= rows) return;
+    const T* xr = x + row * (long)cols;
+    T* yr = y + row * (long)cols;
+    float ss = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = Elem<T>::load1(xr + c);
+        ss = __builtin_fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    __shared__ float part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = (part[0] + part[1]) + (part[2] + part[3]);
+    const float s = fast_rsqrt(ss * inv_cols + eps);
+    if (threadIdx.x == 0 && inv_rms != nullptr) inv_rms[row] = s;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = Elem<T>::load1(xr + c);
+        float wv = Elem<T>::load1(w + c);
+        Elem<T>::store1(yr + c, (v * s) * wv);
+    }
+}
+
+// =================================================================================
+// Backward pass 1, register-resident and persistent.
+//   block = 1024 threads = RG row slots of TPR threads; grid = P workgroups.
+//   Row slot q = blockIdx*RG + rg handles rows q, q + P*RG, q + 2*P*RG, ... and keeps
+//   the dW contributions of its columns in fp32 registers; the next row's x and dy are
+//   requested before the current row is reduced, so loads stay in flight across the
+//   per-row barrier.  At the end the RG slots of a workgroup are added in slot order
+//   through LDS and the workgroup writes row blockIdx of the [P, ld] partial matrix.
+// =================================================================================
+template <typename T, int VEC, int TPR, int ITEMS>
+__global__ void __launch_bounds__(1024)
+rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
+                 const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
+                 long rows, int cols, float inv_cols) {
+    constexpr int BLOCK = 1024;
+    constexpr int RG = BLOCK / TPR;
+    constexpr int WPR = TPR / kWave;
+    constexpr int NW = VEC / 4;
+    constexpr int EPV = VEC / (int)sizeof(T);
+    constexpr int COVER = TPR * ITEMS * EPV;  // columns covered by one row slot (>= cols)
+    static_assert(RG == 1 || COVER * 4 <= 65536, "LDS combine buffer limited to 64 KiB");
+
+    const int tid = threadIdx.x;
+    const int rg = __builtin_amdgcn_readfirstlane(tid / TPR);
+    const int lir = tid - rg * TPR;
+    const long nslots = (long)gridDim.x * RG;
+    const long slot = (long)blockIdx.x * RG + rg;
+    const long n_it = (rows + nslots - 1) / nslots;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+
+    __shared__ float red[2][RG][WPR > 1 ? WPR : 1];
+
+    float acc[ITEMS][EPV];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) acc[i][k] = 0.0f;
+
+    Words<NW> wv[ITEMS];
+    {
+        const rsrc_t rw = make_rsrc(w, row_bytes);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW>(rw, (u32)(lir + i * TPR) * VEC);
+    }
+
+    Words<NW> xv[ITEMS], gv[ITEMS];
+    long row = slot;
+    bool live = row < rows;
+    float s = 0.0f;
+    {
+        const long base = live ? row * (long)cols : 0;
+        const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
+        const rsrc_t rg_ = make_rsrc(dy + base, live ? row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW>(rg_, (u32)(lir + i * TPR) * VEC);
+        if (live) s = inv_rms[row];
+    }
+
+    for (long it = 0; it < n_it; ++it) {
+        // request the next row of this slot (nothing is fetched when there is none)
+        const long nrow = row + nslots;
+        const bool nlive = nrow < rows;
+        Words<NW> nxv[ITEMS], ngv[ITEMS];
+        float ns = 0.0f;
+        {
+            const long nbase = nlive ? nrow * (long)cols : 0;
+            const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
+            const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<NW>(rg_, (u32)(lir + i * TPR) * VEC);
+            if (nlive) ns = inv_rms[nrow];
+        }
+
+        // A = sum dy*w*x over the row; dW += dy*x*s
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            float xf[EPV], gf[EPV], wf[EPV];
+            unpack_vec<T, NW>(xv[i], xf);
+            unpack_vec<T, NW>(gv[i], gf);
+            unpack_vec<T, NW>(wv[i], wf);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                const float t = gf[k] * xf[k];
+                a = __builtin_fmaf(t, wf[k], a);
+                acc[i][k] = __builtin_fmaf(t, s, acc[i][k]);
+            }
+        }
+        a = wave_sum(a);
+        if constexpr (WPR > 1) {
+            const int wir = __builtin_amdgcn_readfirstlane(lir / kWave);
+            const int buf = (int)(it & 1);
+            if ((tid & (kWave - 1)) == 0) red[buf][rg][wir] = a;
+            __syncthreads();
+            float t = 0.0f;
+#pragma unroll
+            for (int k = 0; k < WPR; ++k) t += red[buf][rg][k];
+            a = t;
+        }
+        // dx = s*dy*w - x * (A * s^3 / cols)
+        const float c2 = a * (s * s) * s * inv_cols;
+        {
+            const long base = live ? row * (long)cols : 0;
+            const rsrc_t rd = make_rsrc(dx + base, live ? row_bytes : 0u);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                float xf[EPV], gf[EPV], wf[EPV], o[EPV];
+                unpack_vec<T, NW>(xv[i], xf);
+                unpack_vec<T, NW>(gv[i], gf);
+                unpack_vec<T, NW>(wv[i], wf);
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
+                buf_store<NW>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+        row = nrow; live = nlive; s = ns;
+    }
+
+    // ---- combine the RG row slots in slot order, write this workgroup's partial row ----
+    float* out = dw_part + (long)blockIdx.x * ld;
+    if constexpr (RG == 1) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const int c0 = (lir + i * TPR) * EPV;
+#pragma unroll
+            for (int k = 0; k < EPV; ++k)
+                if (c0 + k < ld) out[c0 + k] = acc[i][k];
+        }
+    } else {
+        __shared__ float dwbuf[COVER];
+        for (int g = 0; g < RG; ++g) {
+            if (rg == g) {
+#pragma unroll
+                for (int i = 0; i < ITEMS; ++i) {
+                    const int c0 = (lir + i * TPR) * EPV;
+#pragma unroll
+                    for (int k = 0; k < EPV; ++k) {
+                        if (g == 0) dwbuf[c0 + k] = acc[i][k];
+                        else dwbuf[c0 + k] += acc[i][k];
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        const int lim = ld < COVER ? ld : COVER;  // ld % 4 == 0 and COVER % 4 == 0
+        for (int c = tid * 4; c < lim; c += BLOCK * 4) {
+            f32x4 v = {dwbuf[c], dwbuf[c + 1], dwbuf[c + 2], dwbuf[c + 3]};
+            *reinterpret_cast<f32x4*>(out + c) = v;
+        }
+    }
+}
+
+// =================================================================================
+// Backward, generic (any cols / alignment): dx per row, then dW partials per column.
+// =================================================================================
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_bwd_dx_generic(T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
+                       const T* __restrict__ w, const float* __restrict__ inv_rms, long rows, int cols,
+                       float inv_cols) {
+    const long row = blockIdx.x;
+    if (row >= rows) return;
+    const T* xr = x + row * (long)cols;
+    const T* gr = dy + row * (long)cols;
+    T* dr = dx + row * (long)cols;
+    const float s = inv_rms[row];
+    float a = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const float t = Elem<T>::load1(gr + c) * Elem<T>::load1(xr + c);
+        a = __builtin_fmaf(t, Elem<T>::load1(w + c), a);
+    }
+    a = wave_sum(a);
+    __shared__ float part[4];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = a;
+    __syncthreads();
+    a = (part[0] + part[1]) + (part[2] + part[3]);
+    const float c2 = a * (s * s) * s * inv_cols;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        const float g = Elem<T>::load1(gr + c) * Elem<T>::load1(w + c);
+        Elem<T>::store1(dr + c, __builtin_fmaf(g, s, -(Elem<T>::load1(xr + c) * c2)));
+    }
+}
+
+// grid = (ceil(cols/256), P); thread owns one column and the rows p, p+P, p+2P, ...
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_bwd_dw_generic(float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
+                       const T* __restrict__ x, const float* __restrict__ inv_rms, long rows, int cols) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int p = blockIdx.y;
+    const int P = gridDim.y;
+    if (c >= cols) return;
+    float acc = 0.0f;
+    for (long r = p; r < rows; r += P) {
+        const float t = Elem<T>::load1(dy + r * (long)cols + c) * Elem<T>::load1(x + r * (long)cols + c);
+        acc = __builtin_fmaf(t, inv_rms[r], acc);
+    }
+    dw_part[(long)p * ld + c] = acc;
+}
+
+// =================================================================================
+// Backward pass 2: dW[c] = sum_p part[p, c] in a fixed order.
+//   block = 256 threads = 16 column quads (64 columns) x 16 row subsets
+//   thread (q, sub) adds rows sub, sub+16, ... ; the 16 subsets are then added in
+//   subset order through LDS.  grid = ceil(cols / 64).
+// =================================================================================
+template <typename TC>
+__global__ void __launch_bounds__(256)
+rmsnorm_dw_reduce(float* __restrict__ dw_f32, TC* __restrict__ dw_cast, const float* __restrict__ part,
+                  int P, int ld, int cols) {
+    const int q = threadIdx.x & 15;
+    const int sub = threadIdx.x >> 4;
+    const int c0 = blockIdx.x * 64 + q * 4;  // < ld because ld % 64 == 0 and grid covers cols
+    f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (c0 < ld) {
+        int p = sub;
+        for (; p + 48 < P; p += 64) {
+            const f32x4 v0 = *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
+            const f32x4 v1 = *reinterpret_cast<const f32x4*>(part + (long)(p + 16) * ld + c0);
+            const f32x4 v2 = *reinterpret_cast<const f32x4*>(part + (long)(p + 32) * ld + c0);
+            const f32x4 v3 = *reinterpret_cast<const f32x4*>(part + (long)(p + 48) * ld + c0);
+            acc += v0; acc += v1; acc += v2; acc += v3;
+        }
+        for (; p < P; p += 16) acc += *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
+    }
+    __shared__ f32x4 sm[16][16];
+    sm[sub][q] = acc;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int qq = threadIdx.x >> 2, k = threadIdx.x & 3;
+        float t = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) t += sm[j][qq][k];
+        const int c = blockIdx.x * 64 + threadIdx.x;
+        if (c < cols) {
+            if (dw_f32 != nullptr) dw_f32[c] = t;
+            if (dw_cast != nullptr) Elem<TC>::store1(dw_cast + c, t);
+        }
+    }
+}
+
+}  // namespace mg

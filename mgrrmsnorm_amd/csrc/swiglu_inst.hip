@@ -1,0 +1,151 @@
+// SwiGLU activation launchers (all element types) and the dW second pass.
+#include "megagemm_hip.h"
+#include "mg_launch.hpp"
+#include "rmsnorm_kernels.hpp"
+#include "swiglu_kernels.hpp"
+
+namespace mg {
+namespace {
+
+// Zero-fill of the partial matrix for rows == 0 (a kernel rather than a memset node, so
+// that the call behaves the same under stream capture).
+__global__ void __launch_bounds__(256) fill_zero_f32(float* __restrict__ p, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+// units handled by one launch stay below 2^31 so that 32-bit indices cannot wrap
+constexpr long kMaxUnitsPerLaunch = 1L << 31;
+
+template <typename T, int UNROLL>
+hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
+    const long nvr = H * (long)sizeof(T) / 16;
+    const long rows_per_launch = kMaxUnitsPerLaunch / nvr;
+    const FastDiv fd = make_fastdiv((uint32_t)nvr);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * nvr);
+        const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
+        swiglu_fwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
+            (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T, int UNROLL>
+hipError_t bwd_vec(void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
+    const long nvr = H * (long)sizeof(T) / 16;
+    const long rows_per_launch = kMaxUnitsPerLaunch / nvr;
+    const FastDiv fd = make_fastdiv((uint32_t)nvr);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * nvr);
+        const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
+        swiglu_bwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
+            (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t fwd_gen(void* h, const void* gu, long M, long H, hipStream_t s) {
+    const long rows_per_launch = kMaxUnitsPerLaunch / H;
+    const FastDiv fd = make_fastdiv((uint32_t)H);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * H);
+        swiglu_fwd_generic<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+            (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t bwd_gen(void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
+    const long rows_per_launch = kMaxUnitsPerLaunch / H;
+    const FastDiv fd = make_fastdiv((uint32_t)H);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * H);
+        swiglu_bwd_generic<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+            (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t fwd_t(bool vec, int unroll, void* h, const void* gu, long M, long H, hipStream_t s) {
+    if (!vec) return fwd_gen<T>(h, gu, M, H, s);
+    switch (unroll) {
+        case 1: return fwd_vec<T, 1>(h, gu, M, H, s);
+        case 2: return fwd_vec<T, 2>(h, gu, M, H, s);
+        case 4: return fwd_vec<T, 4>(h, gu, M, H, s);
+        case 8: return fwd_vec<T, 8>(h, gu, M, H, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename T>
+hipError_t bwd_t(bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M, long H,
+                 hipStream_t s) {
+    if (!vec) return bwd_gen<T>(dgu, dh, gu, M, H, s);
+    switch (unroll) {
+        case 1: return bwd_vec<T, 1>(dgu, dh, gu, M, H, s);
+        case 2: return bwd_vec<T, 2>(dgu, dh, gu, M, H, s);
+        case 4: return bwd_vec<T, 4>(dgu, dh, gu, M, H, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H,
+                             hipStream_t s) {
+    switch (dtype) {
+        case MG_F32: return fwd_t<float>(vec, unroll, h, gu, M, H, s);
+        case MG_F16: return fwd_t<half_t>(vec, unroll, h, gu, M, H, s);
+        case MG_BF16: return fwd_t<bf16_t>(vec, unroll, h, gu, M, H, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M,
+                             long H, hipStream_t s) {
+    switch (dtype) {
+        case MG_F32: return bwd_t<float>(vec, unroll, dgu, dh, gu, M, H, s);
+        case MG_F16: return bwd_t<half_t>(vec, unroll, dgu, dh, gu, M, H, s);
+        case MG_BF16: return bwd_t<bf16_t>(vec, unroll, dgu, dh, gu, M, H, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* part, int P, int ld,
+                            int cols, hipStream_t s) {
+    const dim3 grid((unsigned)((cols + 63) / 64)), block(256);
+    if (dw_cast == nullptr || cast_dtype == MG_F32) {
+        rmsnorm_dw_reduce<float><<<grid, block, 0, s>>>(dw_f32, (float*)dw_cast, part, P, ld, cols);
+    } else if (cast_dtype == MG_F16) {
+        rmsnorm_dw_reduce<half_t><<<grid, block, 0, s>>>(dw_f32, (half_t*)dw_cast, part, P, ld, cols);
+    } else if (cast_dtype == MG_BF16) {
+        rmsnorm_dw_reduce<bf16_t><<<grid, block, 0, s>>>(dw_f32, (bf16_t*)dw_cast, part, P, ld, cols);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_zero(float* p, long n, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    fill_zero_f32<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(p, n);
+    return hipGetLastError();
+}
+
+}  // namespace mg
