@@ -142,7 +142,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
 }
 
-__device__ __forceinline__ float fast_rsqrt(float v) { return __builtin_amdgcn_rsqf(v); }
+// 1/sqrt(v): the hardware estimate (about 1 ulp) refined by one Newton step, so that the
+// per-row scale, which the backward pass uses cubed, is good to about half an ulp.
+__device__ __forceinline__ float fast_rsqrt(float v) {
+    const float y = __builtin_amdgcn_rsqf(v);
+    const float e = __builtin_fmaf(-(v * y), y, 1.0f);  // 1 - v*y^2
+    return __builtin_fmaf(0.5f * y, e, y);
+}
 
 // sigmoid(g) = 1 / (1 + 2^(-g*log2(e))).  For g << 0 the power overflows to +inf and the
 // reciprocal gives +0, the correct limit.

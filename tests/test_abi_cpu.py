@@ -1,0 +1,164 @@
+"""The C ABI without a GPU: the library loads, exports every function that
+include/megagemm_hip.h declares, and rejects bad arguments before touching HIP (no
+compute call is made here)."""
+import ctypes
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "megagemm_hip.h"
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from mgrrmsnorm_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        from mgrrmsnorm_amd import _build
+
+        _build.build()
+    return _lib.load()
+
+
+def _declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(mg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert _declared_functions() == sorted([
+        "mg_abi_version", "mg_last_error", "mg_set_option", "mg_rmsnorm_fwd", "mg_rmsnorm_bwd_workspace",
+        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd"])
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from mgrrmsnorm_amd import _lib
+
+    for name in _declared_functions():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature in _lib.SIGNATURES"
+    assert sorted(_lib.SIGNATURES) == _declared_functions()
+
+
+def test_header_compiles_as_c_and_cxx(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "megagemm_hip.h"\nint main(void){return MG_ABI_VERSION - 1;}\n')
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", f"-I{HEADER.parent}", "-c", str(src), "-o",
+                    str(tmp_path / "t.o")], check=True)
+    subprocess.run(["g++", "-x", "c++", "-Wall", "-Werror", f"-I{HEADER.parent}", "-c", str(src), "-o",
+                    str(tmp_path / "t2.o")], check=True)
+
+
+def test_abi_version(lib):
+    assert lib.mg_abi_version() == 1
+    text = HEADER.read_text()
+    assert re.search(r"#define\s+MG_ABI_VERSION\s+1\b", text)
+
+
+def _err(lib):
+    return lib.mg_last_error().decode()
+
+
+FAKE = 0x1000  # a non-null, 16-byte aligned address that is never dereferenced on these paths
+
+
+def test_rmsnorm_fwd_rejects_bad_arguments(lib):
+    f = lib.mg_rmsnorm_fwd
+    assert f(FAKE, FAKE, FAKE, FAKE, 4, 8, 1e-5, 7, None) == -1 and "dtype" in _err(lib)
+    assert f(FAKE, FAKE, FAKE, FAKE, -1, 8, 1e-5, 0, None) == -1 and "rows" in _err(lib)
+    assert f(FAKE, FAKE, FAKE, FAKE, 4, 0, 1e-5, 0, None) == -1 and "cols" in _err(lib)
+    assert f(FAKE, FAKE, FAKE, FAKE, 4, 1 << 30, 1e-5, 0, None) == -2 and "too large" in _err(lib)
+    assert f(FAKE, FAKE, FAKE, FAKE, 1 << 31, 8, 1e-5, 2, None) == -2
+    assert f(None, FAKE, FAKE, FAKE, 4, 8, 1e-5, 0, None) == -1 and "NULL" in _err(lib)
+    assert f(FAKE, FAKE, FAKE + 1, FAKE, 4, 8, 1e-5, 1, None) == -1 and "aligned" in _err(lib)
+    # rows == 0 is valid and launches nothing (the reference fails with a launch error)
+    assert f(None, None, None, None, 0, 8, 1e-5, 0, None) == 0
+
+
+def test_rmsnorm_bwd_rejects_bad_arguments(lib):
+    f = lib.mg_rmsnorm_bwd
+    ok = dict(rows=4, cols=8, dtype=2, P=2, ld=64)
+    call = lambda **kw: f(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, *(({**ok, **kw})[k] for k in ("rows", "cols", "dtype", "P", "ld")), None)
+    assert call(dtype=9) == -1
+    assert call(P=0) == -1 and "num_partials" in _err(lib)
+    assert call(P=70000) == -1
+    assert call(ld=8) == -1 and "ld" in _err(lib)
+    assert call(ld=4, cols=8) == -1
+    assert call(cols=100, ld=64) == -1
+    assert f(FAKE, None, FAKE, FAKE, FAKE, FAKE, 4, 8, 2, 2, 64, None) == -1 and "dw_partial" in _err(lib)
+    assert f(None, FAKE, FAKE, FAKE, FAKE, FAKE, 4, 8, 2, 2, 64, None) == -1 and "NULL" in _err(lib)
+
+
+def test_dw_reduce_rejects_bad_arguments(lib):
+    f = lib.mg_rmsnorm_dw_reduce
+    assert f(None, None, 0, FAKE, 2, 64, 8, None) == -1 and "dw_f32" in _err(lib)
+    assert f(FAKE, FAKE, 5, FAKE, 2, 64, 8, None) == -1 and "cast_dtype" in _err(lib)
+    assert f(FAKE, None, 0, None, 2, 64, 8, None) == -1
+    assert f(FAKE, None, 0, FAKE, 2, 32, 8, None) == -1
+    assert f(FAKE, None, 0, FAKE, 0, 64, 8, None) == -1
+
+
+def test_workspace_rejects_bad_arguments(lib):
+    P, ld = ctypes.c_int64(-5), ctypes.c_int64(-5)
+    f = lib.mg_rmsnorm_bwd_workspace
+    assert f(4, 8, 3, ctypes.byref(P), ctypes.byref(ld)) == -1
+    assert f(4, 8, 0, None, None) == -1
+    assert f(0, 100, 2, ctypes.byref(P), ctypes.byref(ld)) == 0      # no device needed for rows == 0
+    assert (P.value, ld.value) == (1, 128)
+
+
+def test_swiglu_rejects_bad_arguments(lib):
+    assert lib.mg_swiglu_fwd(FAKE, FAKE, 4, 0, 2, None) == -1 and "H" in _err(lib)
+    assert lib.mg_swiglu_fwd(FAKE, FAKE, -1, 8, 2, None) == -1
+    assert lib.mg_swiglu_fwd(FAKE, FAKE, 4, 8, 4, None) == -1
+    assert lib.mg_swiglu_fwd(None, FAKE, 4, 8, 2, None) == -1
+    assert lib.mg_swiglu_fwd(FAKE, FAKE, 4, 1 << 30, 2, None) == -2
+    assert lib.mg_swiglu_fwd(FAKE, FAKE, 1 << 39, 4, 2, None) == -2
+    assert lib.mg_swiglu_fwd(None, None, 0, 8, 2, None) == 0
+    assert lib.mg_swiglu_bwd(FAKE, None, FAKE, 4, 8, 2, None) == -1
+    assert lib.mg_swiglu_bwd(FAKE, FAKE + 2, FAKE, 4, 8, 0, None) == -1 and "aligned" in _err(lib)
+    assert lib.mg_swiglu_bwd(None, None, None, 0, 8, 1, None) == 0
+
+
+def test_set_option(lib):
+    assert lib.mg_set_option(b"no_such_key", 1) == -1 and "unknown key" in _err(lib)
+    assert lib.mg_set_option(None, 1) == -1
+    for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_items", b"bwd_wg_per_cu", b"swiglu_unroll",
+                b"force_generic"):
+        assert lib.mg_set_option(key, 0) == 0
+
+
+def test_fastdiv_matches_integer_division(tmp_path):
+    """The multiply-high division the SwiGLU kernels index with, compiled for the host and
+    compared with `/` over edge-case divisors and dividends."""
+    src = tmp_path / "fd.cpp"
+    src.write_text(r'''
+#include "mg_divmod.hpp"
+#include <cstdio>
+#include <cstdint>
+int main() {
+    const uint32_t ds[] = {1,2,3,5,7,8,9,10,16,33,100,255,256,257,688,1000,1376,4095,4096,4097,11008,65535,65536,
+                           65537,1000003,(1u<<24)-1,1u<<24,(1u<<30)-1,1u<<30,(1u<<31)-1,1u<<31,(1u<<31)+1,0xFFFFFFFFu};
+    uint64_t x = 88172645463325252ull; long bad = 0, n = 0;
+    for (uint32_t d : ds) {
+        mg::FastDiv f = mg::make_fastdiv(d);
+        const uint32_t fixed[] = {0,1,d-1,d,d+1,2*d-1,2*d,0x7FFFFFFFu,0x80000000u,0xFFFFFFFEu,0xFFFFFFFFu};
+        for (uint32_t v : fixed) { ++n; if (mg::fastdiv(v, f) != v / d) ++bad; }
+        for (int i = 0; i < 200000; ++i) {
+            x ^= x << 13; x ^= x >> 7; x ^= x << 17;
+            uint32_t v = (uint32_t)x; ++n;
+            if (mg::fastdiv(v, f) != v / d) ++bad;
+        }
+    }
+    std::printf("%ld %ld\n", n, bad);
+    return bad != 0;
+}
+''')
+    exe = tmp_path / "fd"
+    subprocess.run(["g++", "-O2", "-std=c++17", f"-I{ROOT / 'mgrrmsnorm_amd' / 'csrc'}", str(src), "-o", str(exe)],
+                   check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout

@@ -1,0 +1,294 @@
+"""RMSNorm parity on the GPU, through the C ABI (ctypes on raw device pointers), against
+the CPU oracle on the same seeded inputs, the committed golden vectors, and -- at the full
+benchmark sizes, where the oracle would take too long -- size-independent properties.
+Tolerances: see tests/gpu_util.py."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as U
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+ALL = ["fp32", "fp16", "bf16"]
+EPS = 1e-6
+
+
+def _dev(*ts):
+    return [t.cuda() for t in ts]
+
+
+# ------------------------------------------------------------------------ golden vectors
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("idx", range(6))
+def test_golden_vectors(golden, dtype, idx):
+    c = golden["rmsnorm"][idx]
+    td = U.DTYPES[dtype]
+    x, dy, w = (torch.tensor(c[k], dtype=torch.float64).to(td) for k in ("x", "dy", "w"))
+    assert (x.double() == torch.tensor(c["x"], dtype=torch.float64)).all()   # exact in every storage type
+    xd, dyd, wd = _dev(x, dy, w)
+    y, s = U.rmsnorm_fwd(xd, wd, c["eps"], dtype)
+    U.assert_matches(y, np.array(c["y"]), dtype, "y")
+    np.testing.assert_allclose(s.cpu().numpy(), np.array(c["inv_rms"]), rtol=1e-6)
+    dx, dw, dwc, _ = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    floor = U.dx_floor(c["x"], c["dy"], c["w"], c["inv_rms"])
+    U.assert_matches(dx, np.array(c["dx"]), dtype, "dx", floor=floor)
+    U.assert_dw(dw, np.array(c["dw"]))
+
+
+# ------------------------------------------------------------------ parity with the oracle
+
+SHAPES = [
+    (4096, 4096),    # benchmark shape (and the reference's README shape)
+    (512, 8192),
+    (300, 768),      # one wave per row, partly filled second vector
+    (257, 2048),
+    (129, 4100),     # row pitch not a multiple of 16 bytes: 8-byte vectors, ragged tail
+    (65, 5120),
+    (33, 16384),
+    (7, 100),
+    (5, 33),         # odd width: element-wise kernels
+    (3, 1),
+    (1, 8),
+    (2, 20000),
+    (3, 33000),      # wider than the register-resident kernels hold for 2-byte types
+    (1000, 12),
+]
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_forward_backward_match_oracle(dtype, rows, cols):
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=42 + rows + cols)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    U.assert_matches(y, y_ref, dtype, f"y {rows}x{cols}")
+    np.testing.assert_allclose(s.cpu().numpy(), s_ref, rtol=1e-6, err_msg="inv_rms")
+    dx, dw, dwc, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    U.assert_matches(dx, dx_ref, dtype, f"dx {rows}x{cols}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    assert torch.isfinite(part[:, :cols]).all(), "a partial dW entry was left unwritten"
+    # grad_weight as the reference returns it: the fp32 sum rounded once to the weight type
+    assert torch.equal(dwc, dw.to(U.DTYPES[dtype]))
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("cols", [768, 2048, 4100, 5120, 16384])
+def test_outlier_rows(dtype, cols):
+    """The hidden-size sweep's data: 1% of x and dy scaled by 100, at a row count the oracle
+    handles in seconds."""
+    rows = 1024
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=7 + cols, outliers=True)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    U.assert_matches(y, y_ref, dtype, "y")
+    dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    U.assert_matches(dx, dx_ref, dtype, "dx", floor=floor)
+    U.assert_dw(dw, dw_ref)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_generic_kernels_match_oracle(dtype):
+    """The element-wise path forced on an aligned shape, and taken naturally for a base
+    pointer that is not 16-byte aligned."""
+    rows, cols = 100, 1024
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=99)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    U.check(U.lib().mg_set_option(b"force_generic", 1))
+    try:
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+        dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    finally:
+        U.check(U.lib().mg_set_option(b"force_generic", 0))
+    U.assert_matches(y, y_ref, dtype, "y (forced generic)")
+    U.assert_matches(dx, dx_ref, dtype, "dx (forced generic)", floor=floor)
+    U.assert_dw(dw, dw_ref)
+
+    # misaligned: a view that starts one element into a larger buffer
+    pad = torch.empty(rows * cols + 1, dtype=U.DTYPES[dtype], device="cuda")
+    xm = pad[1:].view(rows, cols)
+    xm.copy_(xd)
+    assert xm.data_ptr() % 16 != 0
+    y2, s2 = U.rmsnorm_fwd(xm, wd, EPS, dtype)
+    U.assert_matches(y2, y_ref, dtype, "y (misaligned x)")
+    dx2, dw2, _, _ = U.rmsnorm_bwd(dyd, xm, wd, s2, dtype)
+    U.assert_matches(dx2, dx_ref, dtype, "dx (misaligned x)", floor=floor)
+    U.assert_dw(dw2, dw_ref)
+
+
+def test_inv_rms_pointer_may_be_null():
+    x, _, w = U.rmsnorm_inputs(64, 512, "bf16")
+    xd, wd = _dev(x, w)
+    y1, _ = U.rmsnorm_fwd(xd, wd, EPS, "bf16", want_inv_rms=True)
+    y2, s2 = U.rmsnorm_fwd(xd, wd, EPS, "bf16", want_inv_rms=False)
+    assert s2 is None and torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_zero_rows(dtype):
+    td = U.DTYPES[dtype]
+    x = torch.empty((0, 256), dtype=td, device="cuda")
+    w = torch.ones(256, dtype=td, device="cuda")
+    y, s = U.rmsnorm_fwd(x, w, EPS, dtype)
+    assert y.shape == (0, 256) and s.shape == (0,)
+    dx, dw, dwc, _ = U.rmsnorm_bwd(x, x, w, s, dtype)
+    torch.cuda.synchronize()
+    assert dx.shape == (0, 256) and (dw == 0).all() and (dwc == 0).all()
+
+
+def test_zero_input_rows_give_zero_output_and_scaled_gradient():
+    rows, cols, eps = 8, 1024, 1e-4
+    x = torch.zeros((rows, cols), dtype=torch.float32, device="cuda")
+    dy = U.cpu_randn((rows, cols), 5).cuda()
+    w = U.cpu_randn((cols,), 6).cuda()
+    y, s = U.rmsnorm_fwd(x, w, eps, "fp32")
+    assert (y == 0).all()
+    np.testing.assert_allclose(s.cpu().numpy(), 100.0, rtol=1e-6)
+    dx, dw, _, _ = U.rmsnorm_bwd(dy, x, w, s, "fp32")
+    np.testing.assert_allclose(dx.cpu().numpy(), (100.0 * dy * w).cpu().numpy(), rtol=2e-6)
+    assert (dw == 0).all()
+
+
+# --------------------------------------------------------------------------- determinism
+
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 2000, 5120), ("fp32", 777, 1000)])
+def test_dw_is_bit_identical_across_runs(dtype, rows, cols):
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=3)
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    first = None
+    for _ in range(10):
+        dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+        if first is None:
+            first = (dx.clone(), dw.clone())
+        else:
+            assert torch.equal(first[1].view(torch.int32), dw.view(torch.int32)), "dW differs between runs"
+            assert torch.equal(first[0], dx)
+
+
+@pytest.mark.parametrize("P", [1, 3, 64, 1000])
+def test_any_number_of_partials_gives_the_same_gradient(P):
+    rows, cols = 515, 2048
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=11)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "bf16")
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+    dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, "bf16", num_partials=P)
+    U.assert_matches(dx, dx_ref, "bf16", f"dx P={P}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    assert torch.isfinite(part[:, :cols]).all()
+
+
+# ------------------------------------------------- full benchmark sizes: exact properties
+
+def _tiled(block: torch.Tensor, reps: int) -> torch.Tensor:
+    return block.unsqueeze(0).expand(reps, *block.shape).reshape(reps * block.shape[0], block.shape[1]).contiguous()
+
+
+FULL = [
+    ("bf16", 16384, 8192),    # forward+backward configuration
+    ("bf16", 65536, 768),
+    ("fp16", 65536, 2048),
+    ("bf16", 65536, 4100),
+    ("fp16", 65536, 5120),
+    ("bf16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
+]
+
+
+@pytest.mark.parametrize("dtype,rows,cols", FULL)
+def test_full_size_by_row_replication(dtype, rows, cols):
+    """Rows are independent, so a matrix made of one 64-row block repeated must give that
+    block's oracle-checked y and dx in every repetition (bit for bit), and reps x its dW."""
+    blk = 64
+    reps = rows // blk
+    x, dy, w = U.rmsnorm_inputs(blk, cols, dtype, seed=1 + cols, outliers=True)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xb, dyb, wd = _dev(x, dy, w)
+    X, DY = _tiled(xb, reps), _tiled(dyb, reps)
+    y, s = U.rmsnorm_fwd(X, wd, EPS, dtype)
+    U.assert_matches(y[:blk], y_ref, dtype, "y, first block")
+    assert torch.equal(y.view(reps, blk, cols), y[:blk].unsqueeze(0).expand(reps, blk, cols)), "y differs between repetitions"
+    assert torch.equal(s.view(reps, blk), s[:blk].unsqueeze(0).expand(reps, blk))
+    del y
+    dx, dw, _, _ = U.rmsnorm_bwd(DY, X, wd, s, dtype)
+    U.assert_matches(dx[:blk], dx_ref, dtype, "dx, first block", floor=floor)
+    assert torch.equal(dx.view(reps, blk, cols), dx[:blk].unsqueeze(0).expand(reps, blk, cols)), "dx differs between repetitions"
+    U.assert_dw(dw, dw_ref * reps, "dW = reps x block dW")
+
+
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("bf16", 16384, 8192), ("bf16", 65536, 768),
+                                             ("fp32", 4096, 4096)])
+def test_power_of_two_scaling_is_exact(dtype, rows, cols):
+    """Scaling dy (or w in the forward pass) by 2 scales every product and sum by exactly 2
+    in binary floating point, so outputs must scale bit-exactly: a linearity check that
+    needs no oracle and runs at full size.  (Not run for fp16, whose subnormal range --
+    reached by a few outputs near zero -- does not round the same way after doubling.)"""
+    td = U.DTYPES[dtype]
+    g = torch.Generator(device="cuda").manual_seed(5)
+    X = torch.randn((rows, cols), generator=g, device="cuda").to(td)
+    DY = torch.randn((rows, cols), generator=g, device="cuda").to(td)
+    W = (1 + 0.02 * torch.randn((cols,), generator=g, device="cuda")).to(td)
+    y1, s = U.rmsnorm_fwd(X, W, EPS, dtype)
+    y2, _ = U.rmsnorm_fwd(X, W * 2, EPS, dtype)
+    assert torch.equal(y2, y1 * 2)
+    dx1, dw1, _, _ = U.rmsnorm_bwd(DY, X, W, s, dtype)
+    dx2, dw2, _, _ = U.rmsnorm_bwd(DY * 2, X, W, s, dtype)
+    assert torch.equal(dx2, dx1 * 2)
+    assert torch.equal(dw2, dw1 * 2)
+
+
+# ------------------------------------------------------------------- streams and graphs
+
+def test_runs_on_the_stream_it_is_given():
+    rows, cols = 2048, 4096
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=21)
+    xd, dyd, wd = _dev(x, dy, w)
+    y0, s0 = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+    dx0, dw0, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s0, "bf16")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        y1, s1 = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+        dx1, dw1, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s1, "bf16")
+    side.synchronize()
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
+
+
+def test_graph_capture_and_replay():
+    """Forward, backward and the dW reduction captured in one HIP graph; every replay, with
+    eager work and synchronisation in between, must reproduce the eager result."""
+    rows, cols = 1024, 4096
+    dtype, code = "bf16", 2
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=31)
+    xd, dyd, wd = _dev(x, dy, w)
+    P, ld = U.bwd_workspace(rows, cols, dtype)
+    y = torch.empty_like(xd); s = torch.empty(rows, device="cuda"); dx = torch.empty_like(xd)
+    part = torch.empty((P, ld), device="cuda"); dw = torch.empty(cols, device="cuda")
+    L = U.lib()
+
+    def enqueue():
+        st = U.stream()
+        U.check(L.mg_rmsnorm_fwd(y.data_ptr(), s.data_ptr(), xd.data_ptr(), wd.data_ptr(), rows, cols, EPS, code, st))
+        U.check(L.mg_rmsnorm_bwd(dx.data_ptr(), part.data_ptr(), dyd.data_ptr(), xd.data_ptr(), wd.data_ptr(),
+                                 s.data_ptr(), rows, cols, code, P, ld, st))
+        U.check(L.mg_rmsnorm_dw_reduce(dw.data_ptr(), None, 0, part.data_ptr(), P, ld, cols, st))
+
+    enqueue()
+    torch.cuda.synchronize()
+    want = (y.clone(), dx.clone(), dw.clone())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    for i in range(4):
+        xd.mul_(1.0)                      # eager work between replays
+        for t in (y, dx, dw):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[0]) and torch.equal(dx, want[1]) and torch.equal(dw, want[2]), f"replay {i}"
