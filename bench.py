@@ -1,0 +1,352 @@
+#!/usr/bin/env python3
+"""Benchmark of the RMSNorm / SwiGLU path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--launch graph|eager]
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM.  The default workload is the one the headline metric is quoted on:
+RMSNorm forward + backward (three launches: forward, backward pass 1, dW reduction) at
+[4096 x 4096] bf16.  The last line printed on stdout is one JSON object; `value` is
+algorithmic bytes per step / wall time per step over exactly K steps.
+
+Buffers rotate over several independent sets whose total size exceeds the 256 MB
+Infinity Cache, so consecutive steps do not find their inputs cached.
+
+Workloads: rmsnorm_fwd_bwd_4096x4096_bf16 (default), rmsnorm_fwd_4096x4096_fp16,
+rmsnorm_fwd_bwd_16384x8192_bf16, rmsnorm_fwd_bwd_65536x{768,2048,4100,5120,16384}_{bf16,fp16},
+swiglu_fwd_bwd_8192x11008_bf16.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import re
+import sys
+import time
+from pathlib import Path
+
+import torch
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+ESIZE = {"fp32": 4, "fp16": 2, "bf16": 2}
+CODE = {"fp32": 0, "fp16": 1, "bf16": 2}
+TORCH = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
+INFINITY_CACHE_BYTES = 256 << 20
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+# ----------------------------------------------------------------------------- workloads
+
+class RmsNormWorkload:
+    """fwd (+ bwd + dW reduce) on [rows, cols]; inputs N(0,1), w = 1 + 0.02 N(0,1), eps 1e-6."""
+
+    def __init__(self, lib, rows, cols, dtype, backward=True, seed=42):
+        self.lib, self.rows, self.cols, self.dtype, self.backward = lib, rows, cols, dtype, backward
+        e = ESIZE[dtype]
+        self.fwd_bytes = 2 * rows * cols * e + cols * e
+        self.bwd_bytes = 3 * rows * cols * e + cols * e + 4 * cols
+        self.step_bytes = self.fwd_bytes + (self.bwd_bytes if backward else 0)
+        per_set = (4 if backward else 2) * rows * cols * e
+        self.nsets = max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
+        td = TORCH[dtype]
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.w = (1 + 0.02 * torch.randn(cols, generator=g, device="cuda")).to(td)
+        self.sets = []
+        for _ in range(self.nsets):
+            s = {"x": torch.randn((rows, cols), generator=g, device="cuda").to(td)}
+            s["y"] = torch.empty_like(s["x"])
+            s["inv_rms"] = torch.empty(rows, dtype=torch.float32, device="cuda")
+            if backward:
+                s["dy"] = torch.randn((rows, cols), generator=g, device="cuda").to(td)
+                s["dx"] = torch.empty_like(s["x"])
+            self.sets.append(s)
+        if backward:
+            P, ld = ctypes.c_int64(0), ctypes.c_int64(0)
+            rc = lib.mg_rmsnorm_bwd_workspace(rows, cols, CODE[dtype], ctypes.byref(P), ctypes.byref(ld))
+            assert rc == 0, lib.mg_last_error()
+            self.P, self.ld = P.value, ld.value
+            self.partial = torch.empty((self.P, self.ld), dtype=torch.float32, device="cuda")
+            self.dw = torch.empty(cols, dtype=torch.float32, device="cuda")
+        self.kernels = {"rmsnorm_fwd": self.fwd_bytes}
+        if backward:
+            self.kernels["rmsnorm_bwd"] = self.bwd_bytes
+        self.dominant = "rmsnorm_bwd" if backward else "rmsnorm_fwd"
+        self.name = f"rmsnorm_{'fwd_bwd' if backward else 'fwd'}_{rows}x{cols}_{dtype}"
+        self.desc = {"rows": rows, "cols": cols, "eps": 1e-6, "launches_per_step": 3 if backward else 1}
+
+    def _chk(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.mg_last_error().decode())
+
+    def fwd(self, i, st):
+        s = self.sets[i % self.nsets]
+        self._chk(self.lib.mg_rmsnorm_fwd(s["y"].data_ptr(), s["inv_rms"].data_ptr(), s["x"].data_ptr(),
+                                          self.w.data_ptr(), self.rows, self.cols, 1e-6, CODE[self.dtype], st))
+
+    def bwd(self, i, st):
+        s = self.sets[i % self.nsets]
+        self._chk(self.lib.mg_rmsnorm_bwd(s["dx"].data_ptr(), self.partial.data_ptr(), s["dy"].data_ptr(),
+                                          s["x"].data_ptr(), self.w.data_ptr(), s["inv_rms"].data_ptr(), self.rows,
+                                          self.cols, CODE[self.dtype], self.P, self.ld, st))
+
+    def reduce(self, i, st):
+        self._chk(self.lib.mg_rmsnorm_dw_reduce(self.dw.data_ptr(), None, 0, self.partial.data_ptr(), self.P,
+                                                self.ld, self.cols, st))
+
+    def step(self, i, st):
+        self.fwd(i, st)
+        if self.backward:
+            self.bwd(i, st)
+            self.reduce(i, st)
+
+    def kernel(self, name):
+        return {"rmsnorm_fwd": self.fwd, "rmsnorm_bwd": self.bwd}[name]
+
+
+class SwigluWorkload:
+    """Activation fwd + bwd on gu [M, 2H] (N(0,1)) and dh [M, H]."""
+
+    def __init__(self, lib, M, H, dtype, seed=42):
+        self.lib, self.M, self.H, self.dtype = lib, M, H, dtype
+        e = ESIZE[dtype]
+        self.fwd_bytes, self.bwd_bytes = 3 * M * H * e, 5 * M * H * e
+        self.step_bytes = self.fwd_bytes + self.bwd_bytes
+        per_set = 6 * M * H * e
+        self.nsets = max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
+        td = TORCH[dtype]
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        self.sets = []
+        for _ in range(self.nsets):
+            s = {"gu": torch.randn((M, 2 * H), generator=g, device="cuda").to(td),
+                 "dh": torch.randn((M, H), generator=g, device="cuda").to(td)}
+            s["h"] = torch.empty_like(s["dh"])
+            s["dgu"] = torch.empty_like(s["gu"])
+            self.sets.append(s)
+        self.kernels = {"swiglu_fwd": self.fwd_bytes, "swiglu_bwd": self.bwd_bytes}
+        self.dominant = "swiglu_bwd"
+        self.name = f"swiglu_fwd_bwd_{M}x{H}_{dtype}"
+        self.desc = {"M": M, "H": H, "launches_per_step": 2}
+
+    def _chk(self, rc):
+        if rc != 0:
+            raise RuntimeError(self.lib.mg_last_error().decode())
+
+    def fwd(self, i, st):
+        s = self.sets[i % self.nsets]
+        self._chk(self.lib.mg_swiglu_fwd(s["h"].data_ptr(), s["gu"].data_ptr(), self.M, self.H, CODE[self.dtype], st))
+
+    def bwd(self, i, st):
+        s = self.sets[i % self.nsets]
+        self._chk(self.lib.mg_swiglu_bwd(s["dgu"].data_ptr(), s["dh"].data_ptr(), s["gu"].data_ptr(), self.M, self.H,
+                                         CODE[self.dtype], st))
+
+    def step(self, i, st):
+        self.fwd(i, st)
+        self.bwd(i, st)
+
+    def kernel(self, name):
+        return {"swiglu_fwd": self.fwd, "swiglu_bwd": self.bwd}[name]
+
+
+def make_workload(lib, name):
+    m = re.fullmatch(r"rmsnorm_(fwd_bwd|fwd)_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
+    if m:
+        return RmsNormWorkload(lib, int(m.group(2)), int(m.group(3)), m.group(4), backward=m.group(1) == "fwd_bwd")
+    m = re.fullmatch(r"swiglu_fwd_bwd_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
+    if m:
+        return SwigluWorkload(lib, int(m.group(1)), int(m.group(2)), m.group(3))
+    raise SystemExit(f"unknown workload '{name}'")
+
+
+# -------------------------------------------------------------------------------- timing
+
+def stream_ptr():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def time_steps(wl, steps, warmup, launch):
+    """Wall time of exactly `steps` steps, synchronised on both sides. Returns seconds."""
+    for i in range(warmup):
+        wl.step(i, stream_ptr())
+    torch.cuda.synchronize()
+    if launch == "graph":
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            st = stream_ptr()
+            for i in range(steps):
+                wl.step(warmup + i, st)
+        graph.replay()            # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+    st = stream_ptr()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        wl.step(warmup + i, st)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def time_kernel(wl, name, launches=200):
+    """Average duration of one launch of `name`, from HIP events around `launches`
+    back-to-back launches on the launch stream (buffers rotating). Returns seconds."""
+    fn = wl.kernel(name)
+    st = stream_ptr()
+    for i in range(10):
+        fn(i, st)
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for i in range(launches):
+            fn(i, st)
+        b.record()
+        b.synchronize()
+        t = a.elapsed_time(b) * 1e-3 / launches
+        best = t if best is None else min(best, t)
+    return best
+
+
+def committed_traffic(kernel, workload):
+    """HBM bytes per launch from the committed rocprofv3 counter summary, if there is one."""
+    path = ROOT / "profiles" / "pmc_traffic.json"
+    if not path.exists():
+        return None
+    try:
+        return json.loads(path.read_text()).get(f"{kernel}@{workload}", {}).get("traffic_bytes")
+    except (ValueError, AttributeError):
+        return None
+
+
+# -------------------------------------------------------------------------- CPU baseline
+
+def cpu_baseline(wl, budget_s=12.0):
+    """The reference's PyTorch formulation on the host cores, fp32 (its CPU-runnable case),
+    on a bounded sample of the same workload: at most 4096 rows, repeated for ~budget_s."""
+    from oracle import torch_ref  # baseline leg only
+
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(42)
+    if isinstance(wl, RmsNormWorkload):
+        rows = min(wl.rows, 4096)
+        x = torch.randn((rows, wl.cols), generator=g)
+        w = 1 + 0.02 * torch.randn(wl.cols, generator=g)
+        dy = torch.randn((rows, wl.cols), generator=g)
+        if wl.backward:
+            fn = lambda: torch_ref.rmsnorm_fwd_bwd(x, w, dy, 1e-6)
+            nbytes = 5 * rows * wl.cols * 4 + 2 * wl.cols * 4 + 4 * wl.cols
+        else:
+            fn = lambda: torch_ref.rmsnorm_formula(x, w, 1e-6)
+            nbytes = 2 * rows * wl.cols * 4 + wl.cols * 4
+        sample = f"{rows}x{wl.cols} fp32, torch CPU formula" + (" + autograd" if wl.backward else "")
+    else:
+        rows = min(wl.M, 1024)
+        gu = torch.randn((rows, 2 * wl.H), generator=g)
+        dh = torch.randn((rows, wl.H), generator=g)
+        fn = lambda: torch_ref.swiglu_fwd_bwd(gu, dh)
+        nbytes = 8 * rows * wl.H * 4
+        sample = f"{rows}x{wl.H} fp32, torch CPU F.silu(gate)*up + autograd"
+    for _ in range(3):
+        fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 10 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{sample}; median of {len(times)} runs = {med * 1e3:.2f} ms; host has {os.cpu_count()} logical CPUs"}
+
+
+# ---------------------------------------------------------------------------------- main
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="rmsnorm_fwd_bwd_4096x4096_bf16")
+    ap.add_argument("--launch", choices=["graph", "eager", "best"], default="best",
+                    help="how the K timed steps are enqueued: one HIP graph, one by one, or the faster of the two")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copies", type=int, default=0,
+                    help="also launch this many plain copies of one activation tensor (mg_copy_bytes), so that a "
+                         "counter profile of this run holds a kernel of known HBM traffic")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        raise SystemExit("bench.py: this build measures one GPU only (the path has no cross-GPU step); "
+                         "run with --gpus 1")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible")
+
+    from mgrrmsnorm_amd import _lib
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    wl = make_workload(lib, args.workload)
+    log(f"[bench] {wl.name}: {wl.step_bytes / 1e6:.1f} MB algorithmic per step, {wl.nsets} buffer sets, "
+        f"device {torch.cuda.get_device_name(0)}")
+
+    if args.calibrate_copies > 0:
+        first = wl.sets[0]
+        src_key, dst_key = ("x", "y") if "x" in first else ("dh", "h")
+        nbytes = first[src_key].numel() * first[src_key].element_size()
+        for i in range(args.calibrate_copies):
+            s_ = wl.sets[i % wl.nsets]
+            rc = lib.mg_copy_bytes(s_[dst_key].data_ptr(), s_[src_key].data_ptr(), nbytes, stream_ptr())
+            assert rc == 0, lib.mg_last_error()
+        torch.cuda.synchronize()
+        log(f"[bench] calibration: {args.calibrate_copies} copies of {nbytes} bytes (traffic 2 x {nbytes} each)")
+
+    modes = ["graph", "eager"] if args.launch == "best" else [args.launch]
+    wall = {}
+    for mode in modes:
+        wall[mode] = time_steps(wl, args.steps, args.warmup, mode)
+        log(f"[bench] {mode}: {wall[mode] / args.steps * 1e6:.2f} us/step")
+    mode = min(wall, key=wall.get)
+    sec_per_step = wall[mode] / args.steps
+    value = wl.step_bytes / sec_per_step / 1e9
+
+    kern = {}
+    for name, nbytes in wl.kernels.items():
+        t = time_kernel(wl, name)
+        kern[name] = {"us": round(t * 1e6, 3), "GB/s": round(nbytes / t / 1e9, 1), "bytes": nbytes}
+        log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch, {nbytes / t / 1e9:.0f} GB/s")
+    dom = wl.dominant
+    achieved = kern[dom]["GB/s"]
+    roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic(dom, wl.name),
+                "algorithmic_bytes": kern[dom]["bytes"], "avg_launch_us": kern[dom]["us"]}
+
+    out = {
+        "metric": "RMSNorm fwd+bwd HBM GB/s at [4096x4096] bf16" if wl.name == "rmsnorm_fwd_bwd_4096x4096_bf16"
+                  else f"{wl.name} HBM GB/s",
+        "value": round(value, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
+        "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
+        "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
+        "kernels": kern, "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl)
+        log(f"[bench] cpu baseline: {out['cpu_baseline']}")
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

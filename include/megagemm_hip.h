@@ -135,6 +135,14 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
                   void* stream);
 
 /*
+ * Measurement aid with no counterpart in the reference: a plain device-to-device copy of
+ * `bytes` (a multiple of 16; both pointers 16-byte aligned) done by one kernel that moves
+ * one 16-byte vector per thread.  Its HBM traffic is exactly 2*bytes, which makes it the
+ * yardstick for calibrating hardware traffic counters when profiling the other kernels.
+ */
+int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
+
+/*
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
  * calling process.  Keys: "fwd_tpr", "fwd_items", "bwd_tpr", "bwd_items" (threads per
  * row / 16-byte vectors per thread, 0 = automatic), "bwd_wg_per_cu", "swiglu_unroll",

@@ -39,6 +39,7 @@ SIGNATURES = {
     "mg_rmsnorm_dw_reduce": (_int, [_vp, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
     "mg_swiglu_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mg_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
+    "mg_copy_bytes": (_int, [_vp, _vp, _i64, _vp]),
 }
 
 

@@ -281,6 +281,18 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
     return MG_OK;
 }
 
+int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream) {
+    if (bytes < 0 || bytes % 16 != 0 || bytes >= (1LL << 40))
+        return fail(MG_ERR_INVALID_ARG, "mg_copy_bytes: bytes must be a non-negative multiple of 16 below 2^40 (got %lld)",
+                    (long long)bytes);
+    if (bytes == 0) return MG_OK;
+    if (dst == nullptr || src == nullptr || !aligned(dst, 16) || !aligned(src, 16))
+        return fail(MG_ERR_INVALID_ARG, "mg_copy_bytes: dst and src must be 16-byte aligned device pointers");
+    hipError_t e = launch_copy(dst, src, (long)bytes, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip("mg_copy_bytes: launch", e);
+    return MG_OK;
+}
+
 static int check_swiglu(const char* fn, int64_t M, int64_t H, int dtype) {
     if (esize_of(dtype) == 0)
         return fail(MG_ERR_INVALID_ARG, "%s: unknown dtype %d (use 0=fp32, 1=fp16, 2=bf16)", fn, dtype);

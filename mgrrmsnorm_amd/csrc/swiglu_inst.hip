@@ -14,6 +14,13 @@ __global__ void __launch_bounds__(256) fill_zero_f32(float* __restrict__ p, long
     if (i < n) p[i] = 0.0f;
 }
 
+// Plain 16-byte copy, one vector per thread: the yardstick the HBM traffic counters are
+// calibrated against (its traffic is exactly 2 * bytes).
+__global__ void __launch_bounds__(256) copy_vec16(u32x4* __restrict__ dst, const u32x4* __restrict__ src, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 // units handled by one launch stay below 2^31 so that 32-bit indices cannot wrap
 constexpr long kMaxUnitsPerLaunch = 1L << 31;
 
@@ -129,7 +136,7 @@ hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const v
 
 hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* part, int P, int ld,
                             int cols, hipStream_t s) {
-    const dim3 grid((unsigned)((cols + 63) / 64)), block(256);
+    const dim3 grid((unsigned)((cols + kReduceCols - 1) / kReduceCols)), block(256);
     if (dw_cast == nullptr || cast_dtype == MG_F32) {
         rmsnorm_dw_reduce<float><<<grid, block, 0, s>>>(dw_f32, (float*)dw_cast, part, P, ld, cols);
     } else if (cast_dtype == MG_F16) {
@@ -139,6 +146,13 @@ hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const 
     } else {
         return hipErrorInvalidValue;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s) {
+    const long n = bytes / 16;
+    if (n <= 0) return hipSuccess;
+    copy_vec16<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>((u32x4*)dst, (const u32x4*)src, n);
     return hipGetLastError();
 }
 

@@ -8,13 +8,14 @@
 
 namespace mg {
 
+// 16-byte global accesses with the non-temporal hint: every element is touched once.
 __device__ __forceinline__ Words<4> gload4(const void* p) {
-    u32x4 t = *reinterpret_cast<const u32x4*>(p);
+    u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
     Words<4> o; o.v[0] = t.x; o.v[1] = t.y; o.v[2] = t.z; o.v[3] = t.w; return o;
 }
 __device__ __forceinline__ void gstore4(void* p, const Words<4>& w) {
     u32x4 t = {w.v[0], w.v[1], w.v[2], w.v[3]};
-    *reinterpret_cast<u32x4*>(p) = t;
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
 }
 
 // total = M * nvr vectors, nvr = H * sizeof(T) / 16 vectors per half row.

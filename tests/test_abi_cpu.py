@@ -31,7 +31,7 @@ def _declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert _declared_functions() == sorted([
         "mg_abi_version", "mg_last_error", "mg_set_option", "mg_rmsnorm_fwd", "mg_rmsnorm_bwd_workspace",
-        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd"])
+        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd", "mg_copy_bytes"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -121,6 +121,13 @@ def test_swiglu_rejects_bad_arguments(lib):
     assert lib.mg_swiglu_bwd(FAKE, None, FAKE, 4, 8, 2, None) == -1
     assert lib.mg_swiglu_bwd(FAKE, FAKE + 2, FAKE, 4, 8, 0, None) == -1 and "aligned" in _err(lib)
     assert lib.mg_swiglu_bwd(None, None, None, 0, 8, 1, None) == 0
+
+
+def test_copy_bytes_rejects_bad_arguments(lib):
+    assert lib.mg_copy_bytes(FAKE, FAKE, 24, None) == -1 and "multiple of 16" in _err(lib)
+    assert lib.mg_copy_bytes(FAKE, FAKE + 4, 32, None) == -1 and "aligned" in _err(lib)
+    assert lib.mg_copy_bytes(None, FAKE, 32, None) == -1
+    assert lib.mg_copy_bytes(None, None, 0, None) == 0
 
 
 def test_set_option(lib):
