@@ -64,7 +64,7 @@ const char* mg_last_error(void);
  * x, y: [rows, cols] of `dtype`; w: [cols] of the same dtype.  Any cols >= 1 is accepted
  * (the reference requires cols % 4 == 0 for fp32 and cols % 2 == 0 otherwise and skips a
  * remainder).  Base pointers must be aligned to the element size; the fast path is taken
- * when they are 16-byte aligned and cols*sizeof(element) is a multiple of 16 (or of 8).
+ * when they are 4-byte aligned and cols*sizeof(element) is a multiple of 4.
  * Limits: cols * sizeof(element) < 2^31, rows < 2^31.
  */
 int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w,
@@ -144,8 +144,9 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
 
 /*
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
- * calling process.  Keys: "fwd_tpr", "fwd_items", "bwd_tpr", "bwd_items" (threads per
- * row / 16-byte vectors per thread, 0 = automatic), "bwd_wg_per_cu", "swiglu_unroll",
+ * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row), "fwd_items" (target
+ * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
+ * workgroup), "bwd_wg_per_cu", "swiglu_unroll",
  * "force_generic" (1 = always take the unvectorised path).  Returns MG_ERR_INVALID_ARG for
  * an unknown key.  Values that do not fit a given problem are ignored for that call.
  */

@@ -28,8 +28,8 @@ int fail_hip(const char* what, hipError_t e) {
 }
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
-std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_items{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0};
+std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0};
 
 int esize_of(int dtype) {
     switch (dtype) {
@@ -72,45 +72,61 @@ int cu_count(int* out) {
 
 int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 
-// Vector width the register-resident kernels can use for this row pitch and these bases:
-// 16, 8, or 0 (generic kernels).
-int pick_vec(long row_bytes, std::initializer_list<const void*> ptrs) {
-    int v = (row_bytes % 16 == 0) ? 16 : (row_bytes % 8 == 0) ? 8 : 0;
-    if (v == 0) return 0;
+// The register-resident kernels need rows that start and end on 4-byte boundaries
+// (16-byte buffer accesses take any dword-aligned address and are range-checked per dword).
+bool rows_vectorizable(long row_bytes, std::initializer_list<const void*> ptrs) {
+    if (row_bytes % 4 != 0) return false;
     for (const void* p : ptrs)
-        if (p != nullptr && !aligned(p, 16)) return 0;
-    return v;
+        if (p != nullptr && !aligned(p, 4)) return false;
+    return true;
 }
 
-int round_items_fwd(int items) { return items == 7 ? 8 : items; }
+int round_items(int items) { return (items == 5 || items == 7) ? items + 1 : items; }
 
-// Forward: the fewest threads per row that keep a thread at or below `target` vectors.
-bool choose_fwd(long row_bytes, int vec, RowCfg* cfg) {
-    const long nvec = row_bytes / vec;
-    int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
+// Forward: the fewest threads per row that keep a thread at or below two vectors (one
+// vector per thread leaves too few bytes in flight); when the second vector would be mostly
+// empty, half the threads with three vectors each.
+bool choose_fwd(long row_bytes, RowCfg* cfg) {
+    const long nvec = (row_bytes + kVec - 1) / kVec;
+    const int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
     if (tpr_ok(tpr)) {
-        const int need = round_items_fwd(ceil_div(nvec, tpr));
-        if (need <= kFwdMaxItems && fwd_items_ok(need)) { *cfg = {vec, tpr, need}; return true; }
+        const int need = ceil_div(nvec, tpr) == 7 ? 8 : ceil_div(nvec, tpr);
+        if (need <= kFwdMaxItems && fwd_items_ok(need)) { *cfg = {kVec, tpr, need, 0}; return true; }
     }
     const int target = (items > 0 && items <= kFwdMaxItems) ? items : 2;
     for (int t = 64; t <= 1024; t *= 2) {
-        const int need = round_items_fwd(ceil_div(nvec, t));
-        if (need <= target || (t == 1024 && need <= kFwdMaxItems)) { *cfg = {vec, t, need}; return true; }
+        int need = ceil_div(nvec, t);
+        if (need == 7) need = 8;
+        if (need <= target || (t == 1024 && need <= kFwdMaxItems)) {
+            if (need == 2 && t >= 128 && nvec * 10 < (long)t * 2 * 6) { t /= 2; need = ceil_div(nvec, t); }
+            *cfg = {kVec, t, need, 0};
+            return true;
+        }
     }
     return false;
 }
 
-bool choose_bwd(long row_bytes, int esize, int vec, RowCfg* cfg) {
-    const long nvec = row_bytes / vec;
-    int tpr = opt_bwd_tpr.load(), items = opt_bwd_items.load();
+// Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  Measured on MI355X,
+// about 64 KiB of loads in flight per compute unit saturates HBM and more waves than that
+// only add contention, so: the most threads per row (fewest vectors per thread) that still
+// keep (row slots) x (row bytes) x (x and dy) x (current + prefetched row) >= 48 KiB.
+bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
+    const long nvec = (row_bytes + kVec - 1) / kVec;
+    const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
     if (tpr_ok(tpr)) {
-        const int need = ceil_div(nvec, tpr);
-        if (bwd_cfg_ok(esize, vec, tpr, need)) { *cfg = {vec, tpr, need}; return true; }
+        const int need = round_items(ceil_div(nvec, tpr));
+        for (int b : {block, 512, 1024})
+            if (bwd_cfg_ok(esize, tpr, need, b)) { *cfg = {kVec, tpr, need, b}; return true; }
     }
-    const int target = (items > 0 && items <= kBwdMaxItems) ? items : 2;
-    for (int t = 64; t <= 1024; t *= 2) {
-        const int need = ceil_div(nvec, t);
-        if ((need <= target || t == 1024) && bwd_cfg_ok(esize, vec, t, need)) { *cfg = {vec, t, need}; return true; }
+    const int b = (block == 1024) ? 1024 : 512;
+    for (int t = b; t >= 64; t /= 2) {
+        const int need = round_items(ceil_div(nvec, t));
+        const long in_flight = (long)(b / t) * row_bytes * 4;
+        if (in_flight >= 48 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+    }
+    for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
+        const int need = round_items(ceil_div(nvec, t));
+        if (bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
     }
     return false;
 }
@@ -152,9 +168,9 @@ int mg_set_option(const char* key, int value) {
     if (key == nullptr) return fail(MG_ERR_INVALID_ARG, "mg_set_option: key is NULL");
     struct { const char* k; std::atomic<int>* v; } table[] = {
         {"fwd_tpr", &opt_fwd_tpr},       {"fwd_items", &opt_fwd_items},
-        {"bwd_tpr", &opt_bwd_tpr},       {"bwd_items", &opt_bwd_items},
+        {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
-        {"force_generic", &opt_force_generic},
+        {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block},
     };
     for (auto& t : table)
         if (strcmp(t.k, key) == 0) { t.v->store(value); return MG_OK; }
@@ -173,12 +189,9 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_fwd: a pointer is not aligned to its element size");
 
     const long row_bytes = cols * es;
-    RowCfg cfg = {0, 0, 0};
+    RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) {
-        const int vec = pick_vec(row_bytes, {y, x, w});
-        generic = (vec == 0) || !choose_fwd(row_bytes, vec, &cfg);
-    }
+    if (!generic) generic = !rows_vectorizable(row_bytes, {y, x, w}) || !choose_fwd(row_bytes, &cfg);
     const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps};
     hipStream_t s = (hipStream_t)stream;
     hipError_t e = by_dtype(
@@ -199,15 +212,18 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
     int cus = 0;
     rc = cu_count(&cus);
     if (rc != MG_OK) return rc;
-    int per_cu = opt_bwd_wg_per_cu.load();
-    if (per_cu < 1 || per_cu > 8) per_cu = 1;
-    // one persistent workgroup per compute unit; fewer when there are not enough rows
-    // to give every row slot of every workgroup at least one row
+    // one persistent workgroup per compute unit (two when a thread holds 4 or more vectors:
+    // such workgroups carry a whole row each and gain from a second one to overlap with);
+    // fewer when there are not enough rows to give every row slot at least one row
     const int es = esize_of(dtype);
-    RowCfg cfg = {0, 0, 0};
-    const int vec = (cols * es % 16 == 0) ? 16 : (cols * es % 8 == 0) ? 8 : 0;
-    int rg = 1;
-    if (vec != 0 && opt_force_generic.load() == 0 && choose_bwd(cols * es, es, vec, &cfg)) rg = 1024 / cfg.tpr;
+    RowCfg cfg = {0, 0, 0, 0};
+    int rg = 1, dflt_per_cu = 1;
+    if (cols * es % 4 == 0 && opt_force_generic.load() == 0 && choose_bwd(cols * es, es, &cfg)) {
+        rg = cfg.block / cfg.tpr;
+        dflt_per_cu = cfg.items >= 4 ? 2 : 1;
+    }
+    int per_cu = opt_bwd_wg_per_cu.load();
+    if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;
     int64_t p = (int64_t)cus * per_cu;
     const int64_t by_rows = (rows + rg - 1) / rg;
     if (p > by_rows) p = by_rows;
@@ -242,12 +258,9 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: a pointer is not aligned to its element size");
 
     const long row_bytes = cols * es;
-    RowCfg cfg = {0, 0, 0};
+    RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) {
-        const int vec = pick_vec(row_bytes, {dx, dy, x, w});
-        generic = (vec == 0) || !choose_bwd(row_bytes, es, vec, &cfg);
-    }
+    if (!generic) generic = !rows_vectorizable(row_bytes, {dx, dy, x, w}) || !choose_bwd(row_bytes, es, &cfg);
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials};
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },

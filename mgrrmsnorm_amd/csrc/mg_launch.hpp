@@ -8,22 +8,28 @@ namespace mg {
 
 // How a row is spread over threads in the register-resident RMSNorm kernels.
 struct RowCfg {
-    int vec;    // bytes per vector load: 16 or 8
+    int vec;    // bytes per vector load (16)
     int tpr;    // threads per row: 64, 128, 256, 512, 1024
     int items;  // vectors per thread
+    int block;  // backward only: threads per workgroup, 1024 or 512
 };
+
+constexpr int kVec = 16;
 
 // Largest ITEMS instantiated.
 constexpr int kFwdMaxItems = 8;
-constexpr int kBwdMaxItems = 4;
+constexpr int kBwdMaxItems = 8;
 
 // Forward: ITEMS in {1,2,3,4,5,6,8}.
 constexpr bool fwd_items_ok(int items) { return items >= 1 && items <= 8 && items != 7; }
-// Backward: ITEMS in {1,2,3,4}; when several row slots share a workgroup their combine
-// buffer (tpr * items * elements-per-vector floats) must fit 64 KiB of LDS.
-constexpr bool bwd_cfg_ok(int esize, int vec, int tpr, int items) {
-    return items >= 1 && items <= kBwdMaxItems &&
-           (tpr == 1024 || tpr * items * (vec / esize) * 4 <= 65536);
+// Backward: 1024-thread workgroups (128 VGPRs per thread) hold up to 2 vectors per
+// thread without spilling, 512-thread workgroups (256 VGPRs) up to 8 (ITEMS in
+// {1,2,3,4,6,8}).  When several row slots share a workgroup their combine buffer
+// (tpr * items * elements-per-vector floats) must fit 64 KiB of LDS.
+constexpr bool bwd_cfg_ok(int esize, int tpr, int items, int block) {
+    return (block == 1024 || block == 512) && tpr <= block &&
+           items >= 1 && items <= (block == 1024 ? 2 : kBwdMaxItems) && items != 5 && items != 7 &&
+           (tpr == block || tpr * items * (kVec / esize) * 4 <= 65536);
 }
 constexpr bool tpr_ok(int tpr) { return tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024; }
 

@@ -18,37 +18,42 @@ typedef half_t elem_t;
 typedef bf16_t elem_t;
 #endif
 
-template <int VEC, int TPR, int ITEMS>
+template <int TPR, int ITEMS, int BLOCK>
 hipError_t run(const BwdArgs& a, hipStream_t s) {
-    if constexpr (bwd_cfg_ok((int)sizeof(elem_t), VEC, TPR, ITEMS)) {
-        rmsnorm_bwd_rows<elem_t, VEC, TPR, ITEMS><<<dim3((unsigned)a.num_partials), dim3(1024), 0, s>>>(
-            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
-            a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols);
+    if constexpr (bwd_cfg_ok((int)sizeof(elem_t), TPR, ITEMS, BLOCK)) {
+        rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK>
+            <<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
+                (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
+                a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols);
         return hipGetLastError();
     } else {
         return hipErrorInvalidValue;
     }
 }
 
-template <int VEC, int TPR>
+template <int TPR, int BLOCK>
 hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
     switch (items) {
-        case 1: return run<VEC, TPR, 1>(a, s);
-        case 2: return run<VEC, TPR, 2>(a, s);
-        case 3: return run<VEC, TPR, 3>(a, s);
-        case 4: return run<VEC, TPR, 4>(a, s);
+        case 1: return run<TPR, 1, BLOCK>(a, s);
+        case 2: return run<TPR, 2, BLOCK>(a, s);
+        case 3: return run<TPR, 3, BLOCK>(a, s);
+        case 4: return run<TPR, 4, BLOCK>(a, s);
+        case 6: return run<TPR, 6, BLOCK>(a, s);
+        case 8: return run<TPR, 8, BLOCK>(a, s);
         default: return hipErrorInvalidValue;
     }
 }
 
-template <int VEC>
+template <int BLOCK>
 hipError_t by_tpr(int tpr, int items, const BwdArgs& a, hipStream_t s) {
     switch (tpr) {
-        case 64: return by_items<VEC, 64>(items, a, s);
-        case 128: return by_items<VEC, 128>(items, a, s);
-        case 256: return by_items<VEC, 256>(items, a, s);
-        case 512: return by_items<VEC, 512>(items, a, s);
-        case 1024: return by_items<VEC, 1024>(items, a, s);
+        case 64: return by_items<64, BLOCK>(items, a, s);
+        case 128: return by_items<128, BLOCK>(items, a, s);
+        case 256: return by_items<256, BLOCK>(items, a, s);
+        case 512: return by_items<512, BLOCK>(items, a, s);
+        case 1024:
+            if constexpr (BLOCK == 1024) return by_items<1024, BLOCK>(items, a, s);
+            else return hipErrorInvalidValue;
         default: return hipErrorInvalidValue;
     }
 }
@@ -68,8 +73,9 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
                 a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
         return hipGetLastError();
     }
-    if (cfg.vec == 16) return by_tpr<16>(cfg.tpr, cfg.items, a, s);
-    if (cfg.vec == 8) return by_tpr<8>(cfg.tpr, cfg.items, a, s);
+    if (cfg.vec != kVec) return hipErrorInvalidValue;
+    if (cfg.block == 1024) return by_tpr<1024>(cfg.tpr, cfg.items, a, s);
+    if (cfg.block == 512) return by_tpr<512>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;
 }
 

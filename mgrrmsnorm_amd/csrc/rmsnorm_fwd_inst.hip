@@ -65,8 +65,7 @@ hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const Fwd
             1.0f / (float)a.cols);
         return hipGetLastError();
     }
-    if (cfg.vec == 16) return by_tpr<16>(cfg.tpr, cfg.items, a, s);
-    if (cfg.vec == 8) return by_tpr<8>(cfg.tpr, cfg.items, a, s);
+    if (cfg.vec == kVec) return by_tpr<kVec>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;
 }
 

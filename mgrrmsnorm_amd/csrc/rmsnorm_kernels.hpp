@@ -1,14 +1,18 @@
 // RMSNorm forward / backward kernels for gfx950.
 //
 // Register-resident family ("rows" kernels): a row of `cols` elements is split into
-// vectors of VEC bytes; TPR threads (a multiple of the 64-lane wave) share one row and
-// each holds ITEMS vectors of it in VGPRs, vector i of thread t being vector t + i*TPR of
-// the row.  All of a row's loads are issued before the first use.  Row sums are reduced
+// vectors of VEC = 16 bytes; TPR threads (a multiple of the 64-lane wave) share one row
+// and each holds ITEMS vectors of it in VGPRs, vector i of thread t being vector t + i*TPR
+// of the row.  All of a row's loads are issued before the first use.  Row sums are reduced
 // with DPP inside a wave and through a few floats of LDS across the waves of a row.
+// Rows only need 4-byte alignment: buffer_load/store_dwordx4 take any dword-aligned
+// address, and the range check against the row's byte length is made per dword, so a row
+// whose length is not a multiple of 16 simply ends inside its last vector (the lanes and
+// dwords beyond it load 0 and store nothing).
 //
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
-// the row; used when the row pitch is not a multiple of 8 bytes, a base pointer is not
-// 16-byte aligned, or the row does not fit the register-resident family.
+// the row; used when the row pitch or a base pointer is not a multiple of 4 bytes, or the
+// row does not fit the register-resident family.
 #pragma once
 #include "mg_device.hpp"
 
@@ -113,19 +117,19 @@ rmsnorm_fwd_generic(T* __restrict__ y, float* __restrict__ inv_rms, const T* __r
 
 // =================================================================================
 // Backward pass 1, register-resident and persistent.
-//   block = 1024 threads = RG row slots of TPR threads; grid = P workgroups.
+//   block = BLOCK threads (1024 or 512) = RG row slots of TPR threads; grid = P workgroups.
 //   Row slot q = blockIdx*RG + rg handles rows q, q + P*RG, q + 2*P*RG, ... and keeps
 //   the dW contributions of its columns in fp32 registers; the next row's x and dy are
 //   requested before the current row is reduced, so loads stay in flight across the
 //   per-row barrier.  At the end the RG slots of a workgroup are added in slot order
 //   through LDS and the workgroup writes row blockIdx of the [P, ld] partial matrix.
 // =================================================================================
-template <typename T, int VEC, int TPR, int ITEMS>
-__global__ void __launch_bounds__(1024)
+template <typename T, int VEC, int TPR, int ITEMS, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
 rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                  const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
                  long rows, int cols, float inv_cols) {
-    constexpr int BLOCK = 1024;
+    static_assert(BLOCK % TPR == 0 && TPR % kWave == 0, "row slots must tile the workgroup");
     constexpr int RG = BLOCK / TPR;
     constexpr int WPR = TPR / kWave;
     constexpr int NW = VEC / 4;

@@ -133,7 +133,7 @@ def test_copy_bytes_rejects_bad_arguments(lib):
 def test_set_option(lib):
     assert lib.mg_set_option(b"no_such_key", 1) == -1 and "unknown key" in _err(lib)
     assert lib.mg_set_option(None, 1) == -1
-    for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_items", b"bwd_wg_per_cu", b"swiglu_unroll",
+    for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_block", b"bwd_wg_per_cu", b"swiglu_unroll",
                 b"force_generic"):
         assert lib.mg_set_option(key, 0) == 0
 
