@@ -87,9 +87,37 @@ def dtype_code(dtype: torch.dtype) -> int:
             f"Unsupported dtype {dtype}. Use float32, float16, or bfloat16.") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr(device: torch.device) -> int:
     """Raw hipStream_t of torch's current stream on `device`."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)     # no Stream object is built on this path
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class device_of:
+    """Makes the tensor's device current for the enclosed launches, like
+    torch.cuda.device(...) but free when it already is (the common case)."""
+
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, device: torch.device):
+        self.idx = device.index
+        self.prev = -1
+
+    def __enter__(self):
+        cur = torch.cuda.current_device()
+        if self.idx is not None and cur != self.idx:
+            self.prev = cur
+            torch.cuda.set_device(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 def set_option(key: str, value: int) -> None:

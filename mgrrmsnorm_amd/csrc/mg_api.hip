@@ -333,7 +333,7 @@ int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void
     if (!aligned(h, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: a pointer is not aligned to its element size");
     const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(h, 16) && aligned(gu, 16);
-    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(4, 8), h, gu, (long)M, (long)H, (hipStream_t)stream);
+    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(1, 8), h, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_fwd: launch", e);
     return MG_OK;
 }
@@ -350,7 +350,7 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
     const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(dgu, 16) && aligned(dh, 16) &&
                      aligned(gu, 16);
     hipError_t e =
-        launch_swiglu_bwd(dtype, vec, swiglu_unroll(2, 4), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
+        launch_swiglu_bwd(dtype, vec, swiglu_unroll(1, 4), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_bwd: launch", e);
     return MG_OK;
 }

@@ -324,7 +324,7 @@ rmsnorm_bwd_dw_generic(float* __restrict__ dw_part, int ld, const T* __restrict_
 // =================================================================================
 // Backward pass 2: dW[c] = sum_p part[p, c] in a fixed order.
 //   block = 256 threads = 8 column quads (32 columns = one 128-byte line per partial row)
-//   x 32 row subsets; thread (q, sub) adds rows sub, sub+32, ... with four independent
+//   x 32 row subsets; thread (q, sub) adds rows sub, sub+32, ... with eight independent
 //   loads in flight; the 32 subsets are then added in subset order through LDS.
 //   grid = ceil(cols / 32).
 // =================================================================================
@@ -342,12 +342,12 @@ rmsnorm_dw_reduce(float* __restrict__ dw_f32, TC* __restrict__ dw_cast, const fl
     f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
     if (c0 < ld) {
         int p = sub;
-        for (; p + 3 * SUBS < P; p += 4 * SUBS) {
-            const f32x4 v0 = *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
-            const f32x4 v1 = *reinterpret_cast<const f32x4*>(part + (long)(p + SUBS) * ld + c0);
-            const f32x4 v2 = *reinterpret_cast<const f32x4*>(part + (long)(p + 2 * SUBS) * ld + c0);
-            const f32x4 v3 = *reinterpret_cast<const f32x4*>(part + (long)(p + 3 * SUBS) * ld + c0);
-            acc += v0; acc += v1; acc += v2; acc += v3;
+        for (; p + 7 * SUBS < P; p += 8 * SUBS) {   // 8 independent loads in flight per thread
+            f32x4 v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = *reinterpret_cast<const f32x4*>(part + (long)(p + k * SUBS) * ld + c0);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc += v[k];
         }
         for (; p < P; p += SUBS) acc += *reinterpret_cast<const f32x4*>(part + (long)p * ld + c0);
     }

@@ -46,32 +46,59 @@ def _check_pair(input: torch.Tensor, weight: torch.Tensor) -> None:
 
 def rmsnorm_forward(input: torch.Tensor, weight: torch.Tensor, epsilon: float):
     """y = x * rsqrt(mean(x^2) + eps) * w.  Returns [output, inv_rms]."""
-    for t, n in ((input, "input"), (weight, "weight")):
-        _require_gpu(t, n)
-        _require_contiguous(t, n)
-    _check_pair(input, weight)
+    if not (input.is_cuda and weight.is_cuda and input.is_contiguous() and weight.is_contiguous()):
+        for t, n in ((input, "input"), (weight, "weight")):
+            _require_gpu(t, n)
+            _require_contiguous(t, n)
+    if input.dim() != 2 or weight.dim() != 1 or weight.size(0) != input.size(1) \
+            or weight.dtype != input.dtype or weight.device != input.device:
+        _check_pair(input, weight)
     code = _lib.dtype_code(input.dtype)
     rows, cols = input.shape
     if cols < 1:
         raise RuntimeError("hidden size must be >= 1")
     lib = _lib.load()
-    with torch.cuda.device(input.device):
+    dev = input.device
+    with _lib.device_of(dev):
         output = torch.empty_like(input)
-        inv_rms = torch.empty((rows,), dtype=torch.float32, device=input.device)
+        inv_rms = torch.empty((rows,), dtype=torch.float32, device=dev)
         rc = lib.mg_rmsnorm_fwd(output.data_ptr(), inv_rms.data_ptr(), input.data_ptr(), weight.data_ptr(),
-                                rows, cols, float(epsilon), code, _lib.stream_ptr(input.device))
-    _lib.check(rc, "RMSNorm forward")
+                                rows, cols, epsilon, code, _lib.stream_ptr(dev))
+    if rc != 0:
+        _lib.check(rc, "RMSNorm forward")
     return [output, inv_rms]
+
+
+# (device index, rows, cols, dtype code) -> (num_partials, ld); the answer depends on nothing else
+_workspace_shapes: dict = {}
+
+
+def _bwd_workspace(lib, dev, rows, cols, code):
+    key = (dev.index, rows, cols, code)
+    hit = _workspace_shapes.get(key)
+    if hit is None:
+        n_part, ld = ctypes.c_int64(0), ctypes.c_int64(0)
+        _lib.check(lib.mg_rmsnorm_bwd_workspace(rows, cols, code, ctypes.byref(n_part), ctypes.byref(ld)),
+                   "RMSNorm backward (workspace query)")
+        hit = (n_part.value, ld.value)
+        if len(_workspace_shapes) < 4096:
+            _workspace_shapes[key] = hit
+    return hit
 
 
 def rmsnorm_backward_f32(grad_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
                          inv_rms: torch.Tensor):
     """Backward with dW kept in fp32: returns (grad_input, grad_weight_f32, grad_weight_cast)
     where grad_weight_cast has the weight's dtype (it is grad_weight_f32 itself for fp32)."""
-    for t, n in ((grad_output, "grad_output"), (input, "input"), (weight, "weight"), (inv_rms, "inv_rms")):
-        _require_gpu(t, n)
-        _require_contiguous(t, n)
-    _check_pair(input, weight)
+    if not (grad_output.is_cuda and input.is_cuda and weight.is_cuda and inv_rms.is_cuda
+            and grad_output.is_contiguous() and input.is_contiguous() and weight.is_contiguous()
+            and inv_rms.is_contiguous()):
+        for t, n in ((grad_output, "grad_output"), (input, "input"), (weight, "weight"), (inv_rms, "inv_rms")):
+            _require_gpu(t, n)
+            _require_contiguous(t, n)
+    if input.dim() != 2 or weight.dim() != 1 or weight.size(0) != input.size(1) \
+            or weight.dtype != input.dtype or weight.device != input.device:
+        _check_pair(input, weight)
     if grad_output.shape != input.shape or grad_output.dtype != input.dtype:
         raise RuntimeError("grad_output must have the shape and dtype of input")
     if inv_rms.dtype != torch.float32 or inv_rms.dim() != 1 or inv_rms.size(0) != input.size(0):
@@ -80,23 +107,22 @@ def rmsnorm_backward_f32(grad_output: torch.Tensor, input: torch.Tensor, weight:
     rows, cols = input.shape
     lib = _lib.load()
     dev = input.device
-    with torch.cuda.device(dev):
+    with _lib.device_of(dev):
         stream = _lib.stream_ptr(dev)
-        n_part, ld = ctypes.c_int64(0), ctypes.c_int64(0)
-        _lib.check(lib.mg_rmsnorm_bwd_workspace(rows, cols, code, ctypes.byref(n_part), ctypes.byref(ld)),
-                   "RMSNorm backward (workspace query)")
+        n_part, ld = _bwd_workspace(lib, dev, rows, cols, code)
         grad_input = torch.empty_like(input)
-        partial = torch.empty((n_part.value, ld.value), dtype=torch.float32, device=dev)
+        partial = torch.empty((n_part, ld), dtype=torch.float32, device=dev)
         dw_f32 = torch.empty((cols,), dtype=torch.float32, device=dev)
-        dw_cast = dw_f32 if weight.dtype == torch.float32 else torch.empty_like(weight)
-        _lib.check(lib.mg_rmsnorm_bwd(grad_input.data_ptr(), partial.data_ptr(), grad_output.data_ptr(),
-                                      input.data_ptr(), weight.data_ptr(), inv_rms.data_ptr(), rows, cols, code,
-                                      n_part.value, ld.value, stream),
-                   "RMSNorm backward")
-        _lib.check(lib.mg_rmsnorm_dw_reduce(dw_f32.data_ptr(),
-                                            None if dw_cast is dw_f32 else dw_cast.data_ptr(), code,
-                                            partial.data_ptr(), n_part.value, ld.value, cols, stream),
-                   "RMSNorm backward (dW reduction)")
+        dw_cast = dw_f32 if code == _lib.MG_F32 else torch.empty_like(weight)
+        rc = lib.mg_rmsnorm_bwd(grad_input.data_ptr(), partial.data_ptr(), grad_output.data_ptr(),
+                                input.data_ptr(), weight.data_ptr(), inv_rms.data_ptr(), rows, cols, code,
+                                n_part, ld, stream)
+        if rc != 0:
+            _lib.check(rc, "RMSNorm backward")
+        rc = lib.mg_rmsnorm_dw_reduce(dw_f32.data_ptr(), None if dw_cast is dw_f32 else dw_cast.data_ptr(), code,
+                                      partial.data_ptr(), n_part, ld, cols, stream)
+        if rc != 0:
+            _lib.check(rc, "RMSNorm backward (dW reduction)")
     return grad_input, dw_f32, dw_cast
 
 
@@ -117,7 +143,7 @@ def swiglu_forward(gate_up: torch.Tensor, hidden_dim: int) -> torch.Tensor:
     code = _lib.dtype_code(gate_up.dtype)
     M = gate_up.size(0)
     lib = _lib.load()
-    with torch.cuda.device(gate_up.device):
+    with _lib.device_of(gate_up.device):
         out = torch.empty((M, hidden_dim), dtype=gate_up.dtype, device=gate_up.device)
         rc = lib.mg_swiglu_fwd(out.data_ptr(), gate_up.data_ptr(), M, hidden_dim, code,
                                _lib.stream_ptr(gate_up.device))
@@ -137,7 +163,7 @@ def swiglu_backward(grad_out: torch.Tensor, gate_up: torch.Tensor, hidden_dim: i
     code = _lib.dtype_code(gate_up.dtype)
     M = gate_up.size(0)
     lib = _lib.load()
-    with torch.cuda.device(gate_up.device):
+    with _lib.device_of(gate_up.device):
         grad_in = torch.empty_like(gate_up)
         rc = lib.mg_swiglu_bwd(grad_in.data_ptr(), grad_out.data_ptr(), gate_up.data_ptr(), M, hidden_dim, code,
                                _lib.stream_ptr(gate_up.device))

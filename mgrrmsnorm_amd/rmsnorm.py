@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import torch
 import torch.nn as nn
+from torch.autograd.function import once_differentiable
 
 from . import ops
 
@@ -26,10 +27,10 @@ class RMSNormFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-5):
         shape = input.shape
-        if input.dim() < 1:
+        if len(shape) < 1:
             raise RuntimeError("RMSNorm needs at least one dimension")
-        x2d = input.contiguous().reshape(-1, shape[-1])
-        w = weight.contiguous()
+        x2d = (input if input.is_contiguous() else input.contiguous()).view(-1, shape[-1])
+        w = weight if weight.is_contiguous() else weight.contiguous()
         y2d, inv_rms = ops.rmsnorm_forward(x2d, w, epsilon)
         ctx.save_for_backward(x2d, w, inv_rms)
         ctx.epsilon = epsilon
@@ -37,12 +38,13 @@ class RMSNormFunction(torch.autograd.Function):
         return y2d.view(shape)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_output: torch.Tensor):
         x2d, w, inv_rms = ctx.saved_tensors
-        dy2d = grad_output.contiguous().view(-1, grad_output.size(-1))
+        dy2d = (grad_output if grad_output.is_contiguous() else grad_output.contiguous()).view(x2d.shape)
         if dy2d.dtype != x2d.dtype:
             dy2d = dy2d.to(x2d.dtype)
-        dx2d, dw = ops.rmsnorm_backward(dy2d, x2d, w, inv_rms)
+        dx2d, _, dw = ops.rmsnorm_backward_f32(dy2d, x2d, w, inv_rms)
         return dx2d.view(ctx.orig_shape), dw, None
 
 

@@ -1,0 +1,66 @@
+"""Packaging for mgrrmsnorm_amd: `pip install -e .` (or `python setup.py build`) compiles
+libmegagemm_hip.so for gfx950 with hipcc and ships it inside the package, next to the
+ctypes loader.  There is no torch C++ extension to build: the binding is the plain C ABI
+in include/megagemm_hip.h.  (Reference: a CUDAExtension built by nvcc, setup.py:23-41.)
+"""
+import sys
+from pathlib import Path
+
+from setuptools import Command, setup
+from setuptools.command.build_py import build_py
+from setuptools.command.develop import develop
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+
+def _compile_library():
+    from mgrrmsnorm_amd import _build
+
+    print(f"building {_build.LIB_PATH} for {_build.ARCH}")
+    _build.build()
+
+
+class BuildHip(Command):
+    description = "compile libmegagemm_hip.so with hipcc (gfx950)"
+    user_options = []
+
+    def initialize_options(self):
+        pass
+
+    def finalize_options(self):
+        pass
+
+    def run(self):
+        _compile_library()
+
+
+class BuildPyWithHip(build_py):
+    def run(self):
+        _compile_library()
+        super().run()
+
+
+class DevelopWithHip(develop):
+    def run(self):
+        _compile_library()
+        super().run()
+
+
+setup(
+    name="mgrrmsnorm-amd",
+    version="0.1.0",
+    description=("RMSNorm and SwiGLU activation as hand-written HIP kernels for AMD MI355X (gfx950), "
+                 "with the Python surface of MadrasLe/MGRrmsnorm's megagemm package"),
+    long_description=(ROOT / "README.md").read_text(),
+    long_description_content_type="text/markdown",
+    license="MIT",
+    python_requires=">=3.9",
+    install_requires=["torch>=2.0"],
+    extras_require={"dev": ["pytest", "numpy"]},
+    packages=["mgrrmsnorm_amd", "megagemm"],
+    py_modules=["rmsnorm_cuda_ops"],
+    package_data={"mgrrmsnorm_amd": ["libmegagemm_hip.so", "csrc/*.hip", "csrc/*.hpp", "csrc/tools/*.hip"]},
+    data_files=[("include", ["include/megagemm_hip.h"])],
+    cmdclass={"build_hip": BuildHip, "build_py": BuildPyWithHip, "develop": DevelopWithHip},
+)
