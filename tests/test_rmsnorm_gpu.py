@@ -45,11 +45,13 @@ SHAPES = [
     (512, 8192),
     (300, 768),      # one wave per row, partly filled second vector
     (257, 2048),
-    (129, 4100),     # row pitch not a multiple of 16 bytes: 8-byte vectors, ragged tail
+    (129, 4100),     # row pitch 8200 bytes: every other row starts 8 bytes off a 16-byte boundary
+    (67, 4098),      # row pitch 8196 bytes: rows are only 4-byte aligned, the last vector is ragged
+    (31, 8190),
     (65, 5120),
     (33, 16384),
     (7, 100),
-    (5, 33),         # odd width: element-wise kernels
+    (5, 33),         # odd width: element-wise kernels for 2-byte types, vector kernels for fp32
     (3, 1),
     (1, 8),
     (2, 20000),
