@@ -294,3 +294,64 @@ def test_graph_capture_and_replay():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, want[0]) and torch.equal(dx, want[1]) and torch.equal(dw, want[2]), f"replay {i}"
+
+
+# ----------------------------------------------------------------- seeded random shapes
+
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        rows = int(rng.integers(1, 400))
+        cols = int(rng.choice([rng.integers(1, 64), rng.integers(64, 1200), rng.integers(1200, 9000)]))
+        out.append((rows, cols))
+    return out
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_random_shapes_match_oracle(dtype):
+    """36 seeded (rows, cols) pairs per type, odd and ragged widths included: every launch
+    shape the host can choose, both kernel families, and rows that do not fill the grid."""
+    for rows, cols in _random_shapes(36, seed={"fp32": 1, "fp16": 2, "bf16": 3}[dtype]):
+        x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=rows * 7919 + cols)
+        y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+        xd, dyd, wd = _dev(x, dy, w)
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+        U.assert_matches(y, y_ref, dtype, f"y {rows}x{cols}")
+        dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+        U.assert_matches(dx, dx_ref, dtype, f"dx {rows}x{cols}", floor=floor)
+        U.assert_dw(dw, dw_ref, f"dW {rows}x{cols}")
+        assert torch.isfinite(part[:, :cols]).all(), f"partial dW not fully written at {rows}x{cols}"
+
+
+@pytest.mark.parametrize("block,tpr", [(1024, 64), (1024, 256), (1024, 1024), (512, 64), (512, 128), (512, 512)])
+def test_every_backward_workgroup_shape(block, tpr):
+    """Launch shapes the automatic choice does not pick for this size still give the same answer."""
+    rows, cols = 700, 1024                      # 128 vectors per row: 2 per thread at 64 threads per row
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=17)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "bf16")
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+    L = U.lib()
+    U.check(L.mg_set_option(b"bwd_block", block)); U.check(L.mg_set_option(b"bwd_tpr", tpr))
+    try:
+        dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, "bf16")
+    finally:
+        U.check(L.mg_set_option(b"bwd_block", 0)); U.check(L.mg_set_option(b"bwd_tpr", 0))
+    U.assert_matches(dx, dx_ref, "bf16", f"dx block={block} tpr={tpr}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+
+
+@pytest.mark.parametrize("tpr", [64, 128, 256, 512, 1024])
+def test_every_forward_workgroup_shape(tpr):
+    rows, cols = 333, 4096
+    x, _, w = U.rmsnorm_inputs(rows, cols, "fp16", seed=19)
+    y_ref, s_ref, *_ = U.rmsnorm_reference(x, None, w, EPS, "fp16")
+    xd, wd = _dev(x, w)
+    U.check(U.lib().mg_set_option(b"fwd_tpr", tpr))
+    try:
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, "fp16")
+    finally:
+        U.check(U.lib().mg_set_option(b"fwd_tpr", 0))
+    U.assert_matches(y, y_ref, "fp16", f"y tpr={tpr}")
+    np.testing.assert_allclose(s.cpu().numpy(), s_ref, rtol=1e-6)

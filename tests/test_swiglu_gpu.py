@@ -169,3 +169,15 @@ def test_graph_capture_and_replay():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(h, want[0]) and torch.equal(d, want[1]), f"replay {i}"
+
+
+def test_random_shapes_match_oracle():
+    rng = np.random.default_rng(5)
+    for dtype in ALL:
+        for _ in range(20):
+            M = int(rng.integers(1, 300))
+            H = int(rng.choice([rng.integers(1, 40), rng.integers(40, 3000)]))
+            gu, dh = _inputs(M, H, dtype, seed=M * 31 + H, scale=2.0)
+            h_ref, d_ref, floor = U.swiglu_reference(gu, dh, dtype)
+            U.assert_matches(U.swiglu_fwd(gu.cuda(), H, dtype), h_ref, dtype, f"h {M}x{H}")
+            U.assert_matches(U.swiglu_bwd(dh.cuda(), gu.cuda(), H, dtype), d_ref, dtype, f"dgu {M}x{H}", floor=floor)
