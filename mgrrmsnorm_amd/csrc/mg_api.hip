@@ -172,6 +172,7 @@ int mg_set_option(const char* key, int value) {
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block},
     };
+    if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
     for (auto& t : table)
         if (strcmp(t.k, key) == 0) { t.v->store(value); return MG_OK; }
     return fail(MG_ERR_INVALID_ARG, "mg_set_option: unknown key '%s'", key);

@@ -54,6 +54,8 @@ hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s);
 
 // SwiGLU: `vec` = true takes the 16-byte kernels (requires H*sizeof(T) % 16 == 0 and
 // 16-byte aligned bases).  rows*H per launch must stay below 2^31 units (vectors or elements).
+// Upper bound on units per launch (default and maximum 2^31); larger inputs are split by rows.
+void set_swiglu_max_units(long units);
 hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H, hipStream_t s);
 hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M,
                              long H, hipStream_t s);

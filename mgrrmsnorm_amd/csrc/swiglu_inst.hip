@@ -4,6 +4,8 @@
 #include "rmsnorm_kernels.hpp"
 #include "swiglu_kernels.hpp"
 
+#include <atomic>
+
 namespace mg {
 namespace {
 
@@ -22,12 +24,19 @@ __global__ void __launch_bounds__(256) copy_vec16(u32x4* __restrict__ dst, const
 }
 
 // units handled by one launch stay below 2^31 so that 32-bit indices cannot wrap
-constexpr long kMaxUnitsPerLaunch = 1L << 31;
+constexpr long kMaxUnitsPerLaunchDefault = 1L << 31;
+std::atomic<long> g_max_units{kMaxUnitsPerLaunchDefault};
+
+// rows one launch may cover when a row has `units_per_row` units (at least one row)
+long rows_per_launch_for(long units_per_row) {
+    const long r = g_max_units.load(std::memory_order_relaxed) / units_per_row;
+    return r < 1 ? 1 : r;
+}
 
 template <typename T, int UNROLL>
 hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
     const long nvr = H * (long)sizeof(T) / 16;
-    const long rows_per_launch = kMaxUnitsPerLaunch / nvr;
+    const long rows_per_launch = rows_per_launch_for(nvr);
     const FastDiv fd = make_fastdiv((uint32_t)nvr);
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
@@ -44,7 +53,7 @@ hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
 template <typename T, int UNROLL>
 hipError_t bwd_vec(void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
     const long nvr = H * (long)sizeof(T) / 16;
-    const long rows_per_launch = kMaxUnitsPerLaunch / nvr;
+    const long rows_per_launch = rows_per_launch_for(nvr);
     const FastDiv fd = make_fastdiv((uint32_t)nvr);
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
@@ -60,7 +69,7 @@ hipError_t bwd_vec(void* dgu, const void* dh, const void* gu, long M, long H, hi
 
 template <typename T>
 hipError_t fwd_gen(void* h, const void* gu, long M, long H, hipStream_t s) {
-    const long rows_per_launch = kMaxUnitsPerLaunch / H;
+    const long rows_per_launch = rows_per_launch_for(H);
     const FastDiv fd = make_fastdiv((uint32_t)H);
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
@@ -75,7 +84,7 @@ hipError_t fwd_gen(void* h, const void* gu, long M, long H, hipStream_t s) {
 
 template <typename T>
 hipError_t bwd_gen(void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
-    const long rows_per_launch = kMaxUnitsPerLaunch / H;
+    const long rows_per_launch = rows_per_launch_for(H);
     const FastDiv fd = make_fastdiv((uint32_t)H);
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
@@ -113,6 +122,10 @@ hipError_t bwd_t(bool vec, int unroll, void* dgu, const void* dh, const void* gu
 }
 
 }  // namespace
+
+void set_swiglu_max_units(long units) {
+    g_max_units.store(units >= 1 && units <= kMaxUnitsPerLaunchDefault ? units : kMaxUnitsPerLaunchDefault);
+}
 
 hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H,
                              hipStream_t s) {

@@ -199,6 +199,7 @@ FULL = [
     ("bf16", 65536, 4100),
     ("fp16", 65536, 5120),
     ("bf16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
+    ("fp32", 70000, 16388),   # 4.6 GB per tensor, rows 4-byte aligned only: offsets beyond 2^32
 ]
 
 

@@ -181,3 +181,21 @@ def test_random_shapes_match_oracle():
             h_ref, d_ref, floor = U.swiglu_reference(gu, dh, dtype)
             U.assert_matches(U.swiglu_fwd(gu.cuda(), H, dtype), h_ref, dtype, f"h {M}x{H}")
             U.assert_matches(U.swiglu_bwd(dh.cuda(), gu.cuda(), H, dtype), d_ref, dtype, f"dgu {M}x{H}", floor=floor)
+
+
+@pytest.mark.parametrize("limit", [1, 1000, 5000])
+def test_inputs_split_over_several_launches(limit):
+    """Inputs beyond 2^31 units per launch are split by rows; with the limit lowered the same
+    code path runs at a size the oracle can check (vector and element-wise kernels)."""
+    L = U.lib()
+    for dtype, (M, H) in (("bf16", (37, 1376)), ("fp32", (53, 33)), ("fp16", (19, 100))):
+        gu, dh = _inputs(M, H, dtype, seed=limit + M)
+        h_ref, d_ref, floor = U.swiglu_reference(gu, dh, dtype)
+        U.check(L.mg_set_option(b"swiglu_max_units", limit))
+        try:
+            h = U.swiglu_fwd(gu.cuda(), H, dtype)
+            d = U.swiglu_bwd(dh.cuda(), gu.cuda(), H, dtype)
+        finally:
+            U.check(L.mg_set_option(b"swiglu_max_units", 0))
+        U.assert_matches(h, h_ref, dtype, f"h split at {limit}")
+        U.assert_matches(d, d_ref, dtype, f"dgu split at {limit}", floor=floor)
