@@ -191,3 +191,47 @@ def test_state_dict_round_trip_between_module_names():
     n1, n2 = megagemm.RMSNorm(256).cuda(), mgrrmsnorm_amd.RMSNorm(256).cuda()
     n2.load_state_dict(n1.state_dict())
     assert torch.equal(n1(x), n2(x))
+
+
+def test_module_forward_backward_under_graph_capture():
+    """The nn.Module path (allocation through torch's caching allocator, launches through the
+    C ABI) captured into one HIP graph: replays, separated by eager work, reproduce the eager
+    gradients.  This is the way to run small shapes without paying the Python round trip."""
+    from mgrrmsnorm_amd import MegaGemmFunction, RMSNorm
+
+    torch.manual_seed(3)
+    C, H = 2048, 1024
+    norm = RMSNorm(C, 1e-6).cuda().to(torch.bfloat16)
+    x = torch.randn(256, C, device="cuda", dtype=torch.bfloat16, requires_grad=True)
+    proj = torch.randn(C, 2 * H, device="cuda", dtype=torch.bfloat16) * 0.05
+    g = torch.randn(256, H, device="cuda", dtype=torch.bfloat16)
+
+    def step():
+        x.grad = None
+        norm.weight.grad = None
+        out = MegaGemmFunction.apply(norm(x) @ proj, H)
+        out.backward(g)
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                     # warm-up off the default stream, as capture requires
+        for _ in range(3):
+            want_out = step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    want = (want_out.clone(), x.grad.clone(), norm.weight.grad.clone())
+
+    graph = torch.cuda.CUDAGraph()
+    x.grad = None
+    norm.weight.grad = None
+    with torch.cuda.graph(graph):
+        out = step()
+    for i in range(3):
+        torch.zeros(1024, device="cuda").add_(1)       # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want[0]), f"replay {i}: output"
+        assert torch.equal(x.grad, want[1]), f"replay {i}: dx"
+        assert torch.equal(norm.weight.grad, want[2]), f"replay {i}: dW"

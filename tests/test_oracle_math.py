@@ -201,3 +201,56 @@ def test_ulp_distance(oracle):
     assert list(oracle.ulp_distance(a, b, "fp32")) == [1, 0, 0]
     assert oracle.ulp_distance(np.array([0x3F80], np.uint16), np.array([0x3F82], np.uint16), "bf16")[0] == 2
     assert (oracle.to_f32(np.array([0x3F80, 0xC000], np.uint16), "bf16") == [1.0, -2.0]).all()
+
+
+# ------------------------------------------------------------------ hypothesis properties
+
+from hypothesis import given, settings, strategies as st  # noqa: E402
+from hypothesis.extra import numpy as hnp  # noqa: E402
+
+_small = st.floats(min_value=-8, max_value=8, allow_nan=False, width=32)
+
+
+@settings(max_examples=60, deadline=None)
+@given(hnp.arrays(np.float32, st.tuples(st.integers(1, 5), st.integers(1, 40)), elements=_small))
+def test_silu_odd_part_identity(oracle, g):
+    """silu(g) - silu(-g) = g, so h(g, u) - h(-g, u) = g*u for any up value: fails if the
+    sigmoid is evaluated at the wrong sign or the halves are swapped."""
+    u = np.full_like(g, 1.5)
+    hp = oracle.swiglu_fwd_f64(np.concatenate([g, u], axis=1))
+    hm = oracle.swiglu_fwd_f64(np.concatenate([-g, u], axis=1))
+    np.testing.assert_allclose(hp - hm, g.astype(np.float64) * 1.5, rtol=1e-12, atol=1e-12)
+
+
+@settings(max_examples=60, deadline=None)
+@given(hnp.arrays(np.float32, st.tuples(st.integers(1, 4), st.integers(2, 48)), elements=_small),
+       st.integers(0, 10 ** 6))
+def test_rmsnorm_row_has_unit_mean_square(oracle, x, seed):
+    """With w = 1 and eps = 0 every output row has mean square exactly 1 (rows of zeros aside)."""
+    x = x + np.float32(0.125) * np.float32(1 + seed % 3)          # keep rows away from all-zero
+    y, s = oracle.rmsnorm_fwd_f64(x, np.ones(x.shape[1], np.float32), 0.0)
+    keep = np.abs(x).max(-1) > 0
+    np.testing.assert_allclose((y[keep] ** 2).mean(-1), 1.0, rtol=1e-12)
+
+
+@settings(max_examples=40, deadline=None)
+@given(hnp.arrays(np.float32, st.tuples(st.integers(1, 4), st.integers(2, 32)), elements=_small))
+def test_rmsnorm_gradient_matches_finite_difference(oracle, x):
+    """Directional derivative of L = sum(y*dy) along a fixed direction, by central differences
+    in double precision, against <dx, direction> from the oracle's backward."""
+    rows, cols = x.shape
+    rng = np.random.default_rng(rows * 100 + cols)
+    w = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    d = rng.standard_normal((rows, cols))
+    eps = 1e-2
+
+    def loss(xx):
+        xx = np.asarray(xx, np.float64)
+        s = 1 / np.sqrt((xx ** 2).mean(-1, keepdims=True) + eps)
+        return float((xx * s * w * dy).sum())
+
+    h = 1e-6
+    fd = (loss(x + h * d) - loss(x - h * d)) / (2 * h)
+    dx, _ = oracle.rmsnorm_bwd_f64(dy, x, w, eps)
+    assert fd == pytest.approx(float((dx * d).sum()), rel=1e-5, abs=1e-6)
