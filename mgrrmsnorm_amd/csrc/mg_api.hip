@@ -29,7 +29,15 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1};
+
+// Consecutive logical workgroups one die handles at a time in the one-shot streaming
+// kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
+constexpr int kXcdGroupStreaming = 32;
+int xcd_group_or(int dflt) {
+    const int v = opt_xcd_group.load();
+    return v < 0 ? dflt : v;
+}
 
 int esize_of(int dtype) {
     switch (dtype) {
@@ -170,7 +178,7 @@ int mg_set_option(const char* key, int value) {
         {"fwd_tpr", &opt_fwd_tpr},       {"fwd_items", &opt_fwd_items},
         {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
-        {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block},
+        {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
     };
     if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
     for (auto& t : table)
@@ -193,7 +201,7 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
     if (!generic) generic = !rows_vectorizable(row_bytes, {y, x, w}) || !choose_fwd(row_bytes, &cfg);
-    const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps};
+    const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps, xcd_group_or(kXcdGroupStreaming)};
     hipStream_t s = (hipStream_t)stream;
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_fwd<float>(cfg, generic, a, s); },
@@ -262,7 +270,10 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
     if (!generic) generic = !rows_vectorizable(row_bytes, {dx, dy, x, w}) || !choose_bwd(row_bytes, es, &cfg);
-    const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials};
+    // the persistent grid already walks the rows in order; regrouping its workgroups by die
+    // measured within +-2 % either way, so it stays off unless asked for
+    const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,
+                       xcd_group_or(0)};
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },
         [&] { return launch_rmsnorm_bwd<half_t>(cfg, generic, a, s); },
@@ -334,7 +345,7 @@ int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void
     if (!aligned(h, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: a pointer is not aligned to its element size");
     const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(h, 16) && aligned(gu, 16);
-    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(1, 8), h, gu, (long)M, (long)H, (hipStream_t)stream);
+    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(1, 8), xcd_group_or(kXcdGroupStreaming), h, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_fwd: launch", e);
     return MG_OK;
 }
@@ -351,7 +362,7 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
     const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(dgu, 16) && aligned(dh, 16) &&
                      aligned(gu, 16);
     hipError_t e =
-        launch_swiglu_bwd(dtype, vec, swiglu_unroll(1, 4), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
+        launch_swiglu_bwd(dtype, vec, swiglu_unroll(1, 4), xcd_group_or(kXcdGroupStreaming), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_bwd: launch", e);
     return MG_OK;
 }

@@ -36,10 +36,12 @@ constexpr bool tpr_ok(int tpr) { return tpr == 64 || tpr == 128 || tpr == 256 ||
 struct FwdArgs {
     void* y; float* inv_rms; const void* x; const void* w;
     long rows; int cols; float eps;
+    int xcd_group;  // see xcd_remap(); 0 = workgroup ids used as they come
 };
 struct BwdArgs {
     void* dx; float* dw_part; int ld; const void* dy; const void* x; const void* w; const float* inv_rms;
     long rows; int cols; int num_partials;
+    int xcd_group;
 };
 
 // One set of launchers per element type (T = float, _Float16, __bf16), each defined in
@@ -56,8 +58,9 @@ hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s);
 // 16-byte aligned bases).  rows*H per launch must stay below 2^31 units (vectors or elements).
 // Upper bound on units per launch (default and maximum 2^31); larger inputs are split by rows.
 void set_swiglu_max_units(long units);
-hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H, hipStream_t s);
-hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M,
-                             long H, hipStream_t s);
+hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, int xcd_group, void* h, const void* gu, long M, long H,
+                             hipStream_t s);
+hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, int xcd_group, void* dgu, const void* dh, const void* gu,
+                             long M, long H, hipStream_t s);
 
 }  // namespace mg

@@ -24,7 +24,7 @@ hipError_t run(const BwdArgs& a, hipStream_t s) {
         rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK>
             <<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
                 (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
-                a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols);
+                a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);
         return hipGetLastError();
     } else {
         return hipErrorInvalidValue;

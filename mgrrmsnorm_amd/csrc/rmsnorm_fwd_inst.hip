@@ -25,7 +25,7 @@ hipError_t run(const FwdArgs& a, hipStream_t s) {
     const long grid = (a.rows + RPB - 1) / RPB;
     rmsnorm_fwd_rows<elem_t, VEC, TPR, ITEMS><<<dim3((unsigned)grid), dim3(BLOCK), 0, s>>>(
         (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
-        1.0f / (float)a.cols);
+        1.0f / (float)a.cols, a.xcd_group);
     return hipGetLastError();
 }
 

@@ -26,7 +26,7 @@ namespace mg {
 template <typename T, int VEC, int TPR, int ITEMS>
 __global__ void __launch_bounds__((TPR > 256 ? TPR : 256))
 rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
-                 const T* __restrict__ w, long rows, int cols, float eps, float inv_cols) {
+                 const T* __restrict__ w, long rows, int cols, float eps, float inv_cols, int xcd_group) {
     constexpr int BLOCK = TPR > 256 ? TPR : 256;
     constexpr int RPB = BLOCK / TPR;
     constexpr int WPR = TPR / kWave;
@@ -36,7 +36,7 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
     const int tid = threadIdx.x;
     const int rg = __builtin_amdgcn_readfirstlane(tid / TPR);  // row slot inside the workgroup
     const int lir = tid - rg * TPR;                            // lane inside the row
-    const long row = (long)blockIdx.x * RPB + rg;
+    const long row = xcd_remap(blockIdx.x, gridDim.x, xcd_group) * RPB + rg;
     const bool live = row < rows;
     const u32 row_bytes = (u32)cols * (u32)sizeof(T);
     const long base = live ? row * (long)cols : 0;
@@ -118,17 +118,17 @@ rmsnorm_fwd_generic(T* __restrict__ y, float* __restrict__ inv_rms, const T* __r
 // =================================================================================
 // Backward pass 1, register-resident and persistent.
 //   block = BLOCK threads (1024 or 512) = RG row slots of TPR threads; grid = P workgroups.
-//   Row slot q = blockIdx*RG + rg handles rows q, q + P*RG, q + 2*P*RG, ... and keeps
+//   Row slot q = wg*RG + rg (wg = the workgroup's logical id) handles rows q, q + P*RG, q + 2*P*RG, ... and keeps
 //   the dW contributions of its columns in fp32 registers; the next row's x and dy are
 //   requested before the current row is reduced, so loads stay in flight across the
 //   per-row barrier.  At the end the RG slots of a workgroup are added in slot order
-//   through LDS and the workgroup writes row blockIdx of the [P, ld] partial matrix.
+//   through LDS and the workgroup writes row wg of the [P, ld] partial matrix.
 // =================================================================================
 template <typename T, int VEC, int TPR, int ITEMS, int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
 rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                  const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
-                 long rows, int cols, float inv_cols) {
+                 long rows, int cols, float inv_cols, int xcd_group) {
     static_assert(BLOCK % TPR == 0 && TPR % kWave == 0, "row slots must tile the workgroup");
     constexpr int RG = BLOCK / TPR;
     constexpr int WPR = TPR / kWave;
@@ -141,7 +141,8 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
     const int rg = __builtin_amdgcn_readfirstlane(tid / TPR);
     const int lir = tid - rg * TPR;
     const long nslots = (long)gridDim.x * RG;
-    const long slot = (long)blockIdx.x * RG + rg;
+    const long wg = xcd_remap(blockIdx.x, gridDim.x, xcd_group);  // logical workgroup: owns partial row wg
+    const long slot = wg * RG + rg;
     const long n_it = (rows + nslots - 1) / nslots;
     const u32 row_bytes = (u32)cols * (u32)sizeof(T);
 
@@ -240,7 +241,7 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
     }
 
     // ---- combine the RG row slots in slot order, write this workgroup's partial row ----
-    float* out = dw_part + (long)blockIdx.x * ld;
+    float* out = dw_part + wg * ld;
     if constexpr (RG == 1) {
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {

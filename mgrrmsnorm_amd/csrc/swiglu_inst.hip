@@ -34,7 +34,7 @@ long rows_per_launch_for(long units_per_row) {
 }
 
 template <typename T, int UNROLL>
-hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
+hipError_t fwd_vec(int xg, void* h, const void* gu, long M, long H, hipStream_t s) {
     const long nvr = H * (long)sizeof(T) / 16;
     const long rows_per_launch = rows_per_launch_for(nvr);
     const FastDiv fd = make_fastdiv((uint32_t)nvr);
@@ -43,7 +43,7 @@ hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
         const uint32_t total = (uint32_t)(m * nvr);
         const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
         swiglu_fwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
-            (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+            (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd, xg);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -51,7 +51,7 @@ hipError_t fwd_vec(void* h, const void* gu, long M, long H, hipStream_t s) {
 }
 
 template <typename T, int UNROLL>
-hipError_t bwd_vec(void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
+hipError_t bwd_vec(int xg, void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
     const long nvr = H * (long)sizeof(T) / 16;
     const long rows_per_launch = rows_per_launch_for(nvr);
     const FastDiv fd = make_fastdiv((uint32_t)nvr);
@@ -60,7 +60,7 @@ hipError_t bwd_vec(void* dgu, const void* dh, const void* gu, long M, long H, hi
         const uint32_t total = (uint32_t)(m * nvr);
         const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
         swiglu_bwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
-            (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
+            (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd, xg);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -98,25 +98,25 @@ hipError_t bwd_gen(void* dgu, const void* dh, const void* gu, long M, long H, hi
 }
 
 template <typename T>
-hipError_t fwd_t(bool vec, int unroll, void* h, const void* gu, long M, long H, hipStream_t s) {
+hipError_t fwd_t(bool vec, int unroll, int xg, void* h, const void* gu, long M, long H, hipStream_t s) {
     if (!vec) return fwd_gen<T>(h, gu, M, H, s);
     switch (unroll) {
-        case 1: return fwd_vec<T, 1>(h, gu, M, H, s);
-        case 2: return fwd_vec<T, 2>(h, gu, M, H, s);
-        case 4: return fwd_vec<T, 4>(h, gu, M, H, s);
-        case 8: return fwd_vec<T, 8>(h, gu, M, H, s);
+        case 1: return fwd_vec<T, 1>(xg, h, gu, M, H, s);
+        case 2: return fwd_vec<T, 2>(xg, h, gu, M, H, s);
+        case 4: return fwd_vec<T, 4>(xg, h, gu, M, H, s);
+        case 8: return fwd_vec<T, 8>(xg, h, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }
 
 template <typename T>
-hipError_t bwd_t(bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M, long H,
+hipError_t bwd_t(bool vec, int unroll, int xg, void* dgu, const void* dh, const void* gu, long M, long H,
                  hipStream_t s) {
     if (!vec) return bwd_gen<T>(dgu, dh, gu, M, H, s);
     switch (unroll) {
-        case 1: return bwd_vec<T, 1>(dgu, dh, gu, M, H, s);
-        case 2: return bwd_vec<T, 2>(dgu, dh, gu, M, H, s);
-        case 4: return bwd_vec<T, 4>(dgu, dh, gu, M, H, s);
+        case 1: return bwd_vec<T, 1>(xg, dgu, dh, gu, M, H, s);
+        case 2: return bwd_vec<T, 2>(xg, dgu, dh, gu, M, H, s);
+        case 4: return bwd_vec<T, 4>(xg, dgu, dh, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -127,22 +127,22 @@ void set_swiglu_max_units(long units) {
     g_max_units.store(units >= 1 && units <= kMaxUnitsPerLaunchDefault ? units : kMaxUnitsPerLaunchDefault);
 }
 
-hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, void* h, const void* gu, long M, long H,
+hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, int xg, void* h, const void* gu, long M, long H,
                              hipStream_t s) {
     switch (dtype) {
-        case MG_F32: return fwd_t<float>(vec, unroll, h, gu, M, H, s);
-        case MG_F16: return fwd_t<half_t>(vec, unroll, h, gu, M, H, s);
-        case MG_BF16: return fwd_t<bf16_t>(vec, unroll, h, gu, M, H, s);
+        case MG_F32: return fwd_t<float>(vec, unroll, xg, h, gu, M, H, s);
+        case MG_F16: return fwd_t<half_t>(vec, unroll, xg, h, gu, M, H, s);
+        case MG_BF16: return fwd_t<bf16_t>(vec, unroll, xg, h, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }
 
-hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, void* dgu, const void* dh, const void* gu, long M,
-                             long H, hipStream_t s) {
+hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, int xg, void* dgu, const void* dh, const void* gu,
+                             long M, long H, hipStream_t s) {
     switch (dtype) {
-        case MG_F32: return bwd_t<float>(vec, unroll, dgu, dh, gu, M, H, s);
-        case MG_F16: return bwd_t<half_t>(vec, unroll, dgu, dh, gu, M, H, s);
-        case MG_BF16: return bwd_t<bf16_t>(vec, unroll, dgu, dh, gu, M, H, s);
+        case MG_F32: return bwd_t<float>(vec, unroll, xg, dgu, dh, gu, M, H, s);
+        case MG_F16: return bwd_t<half_t>(vec, unroll, xg, dgu, dh, gu, M, H, s);
+        case MG_BF16: return bwd_t<bf16_t>(vec, unroll, xg, dgu, dh, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -21,9 +21,9 @@ __device__ __forceinline__ void gstore4(void* p, const Words<4>& w) {
 // total = M * nvr vectors, nvr = H * sizeof(T) / 16 vectors per half row.
 template <typename T, int UNROLL>
 __global__ void __launch_bounds__(256)
-swiglu_fwd_vec(T* __restrict__ h, const T* __restrict__ gu, uint32_t total, FastDiv nvr) {
+swiglu_fwd_vec(T* __restrict__ h, const T* __restrict__ gu, uint32_t total, FastDiv nvr, int xcd_group) {
     constexpr int EPV = 16 / (int)sizeof(T);
-    const uint32_t v0 = blockIdx.x * (256u * UNROLL) + threadIdx.x;
+    const uint32_t v0 = (uint32_t)xcd_remap(blockIdx.x, gridDim.x, xcd_group) * (256u * UNROLL) + threadIdx.x;
     const char* in = reinterpret_cast<const char*>(gu);
     char* out = reinterpret_cast<char*>(h);
 
@@ -57,9 +57,9 @@ swiglu_fwd_vec(T* __restrict__ h, const T* __restrict__ gu, uint32_t total, Fast
 template <typename T, int UNROLL>
 __global__ void __launch_bounds__(256)
 swiglu_bwd_vec(T* __restrict__ dgu, const T* __restrict__ dh, const T* __restrict__ gu, uint32_t total,
-               FastDiv nvr) {
+               FastDiv nvr, int xcd_group) {
     constexpr int EPV = 16 / (int)sizeof(T);
-    const uint32_t v0 = blockIdx.x * (256u * UNROLL) + threadIdx.x;
+    const uint32_t v0 = (uint32_t)xcd_remap(blockIdx.x, gridDim.x, xcd_group) * (256u * UNROLL) + threadIdx.x;
     const char* in = reinterpret_cast<const char*>(gu);
     const char* din = reinterpret_cast<const char*>(dh);
     char* out = reinterpret_cast<char*>(dgu);
