@@ -146,7 +146,8 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row), "fwd_items" (target
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
- * workgroup), "bwd_wg_per_cu", "swiglu_unroll",
+ * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
+ * the current one; -1 = automatic), "swiglu_unroll",
  * "force_generic" (1 = always take the unvectorised path), "xcd_group" (consecutive workgroups
  * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
  * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for

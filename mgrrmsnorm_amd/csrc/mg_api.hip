@@ -29,7 +29,7 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1};
 
 // Consecutive logical workgroups one die handles at a time in the one-shot streaming
 // kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
@@ -126,7 +126,7 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         for (int b : {block, 512, 1024})
             if (bwd_cfg_ok(esize, tpr, need, b)) { *cfg = {kVec, tpr, need, b}; return true; }
     }
-    const int b = (block == 1024) ? 1024 : 512;
+    for (int b : {block == 1024 ? 1024 : 512, 512}) {
     for (int t = b; t >= 64; t /= 2) {
         const int need = round_items(ceil_div(nvec, t));
         const long in_flight = (long)(b / t) * row_bytes * 4;
@@ -135,6 +135,7 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
         const int need = round_items(ceil_div(nvec, t));
         if (bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+    }
     }
     return false;
 }
@@ -179,6 +180,7 @@ int mg_set_option(const char* key, int value) {
         {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
+        {"bwd_prefetch", &opt_bwd_prefetch},
     };
     if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
     for (auto& t : table)
@@ -221,15 +223,16 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
     int cus = 0;
     rc = cu_count(&cus);
     if (rc != MG_OK) return rc;
-    // one persistent workgroup per compute unit (two when a thread holds 4 or more vectors:
-    // such workgroups carry a whole row each and gain from a second one to overlap with);
+    // one persistent workgroup per compute unit; four when a thread holds 4 or more vectors:
+    // such kernels keep no prefetched copy of the next row (registers) and rely on the other
+    // workgroups of the compute unit to cover the wait for it;
     // fewer when there are not enough rows to give every row slot at least one row
     const int es = esize_of(dtype);
     RowCfg cfg = {0, 0, 0, 0};
     int rg = 1, dflt_per_cu = 1;
     if (cols * es % 4 == 0 && opt_force_generic.load() == 0 && choose_bwd(cols * es, es, &cfg)) {
         rg = cfg.block / cfg.tpr;
-        dflt_per_cu = cfg.items >= 4 ? 2 : 1;
+        dflt_per_cu = cfg.items >= 4 ? 4 : 1;
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;
@@ -273,7 +276,7 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,
-                       xcd_group_or(0)};
+                       xcd_group_or(0), opt_bwd_prefetch.load() < 0 ? cfg.items < 4 : opt_bwd_prefetch.load() != 0};
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },
         [&] { return launch_rmsnorm_bwd<half_t>(cfg, generic, a, s); },

@@ -42,6 +42,7 @@ struct BwdArgs {
     void* dx; float* dw_part; int ld; const void* dy; const void* x; const void* w; const float* inv_rms;
     long rows; int cols; int num_partials;
     int xcd_group;
+    bool prefetch;  // request row i+1 before reducing row i (costs a second copy of the row in VGPRs)
 };
 
 // One set of launchers per element type (T = float, _Float16, __bf16), each defined in

@@ -21,8 +21,9 @@ typedef bf16_t elem_t;
 template <int TPR, int ITEMS, int BLOCK>
 hipError_t run(const BwdArgs& a, hipStream_t s) {
     if constexpr (bwd_cfg_ok((int)sizeof(elem_t), TPR, ITEMS, BLOCK)) {
-        rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK>
-            <<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
+        auto kernel = a.prefetch ? rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK, true>
+                                 : rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK, false>;
+        kernel<<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
                 (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
                 a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);
         return hipGetLastError();

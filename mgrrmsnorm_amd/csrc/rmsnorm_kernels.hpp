@@ -124,7 +124,7 @@ rmsnorm_fwd_generic(T* __restrict__ y, float* __restrict__ inv_rms, const T* __r
 //   per-row barrier.  At the end the RG slots of a workgroup are added in slot order
 //   through LDS and the workgroup writes row wg of the [P, ld] partial matrix.
 // =================================================================================
-template <typename T, int VEC, int TPR, int ITEMS, int BLOCK>
+template <typename T, int VEC, int TPR, int ITEMS, int BLOCK, bool PREFETCH>
 __global__ void __launch_bounds__(BLOCK)
 rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                  const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
@@ -177,12 +177,12 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
     }
 
     for (long it = 0; it < n_it; ++it) {
-        // request the next row of this slot (nothing is fetched when there is none)
         const long nrow = row + nslots;
         const bool nlive = nrow < rows;
-        Words<NW> nxv[ITEMS], ngv[ITEMS];
+        Words<NW> nxv[PREFETCH ? ITEMS : 1], ngv[PREFETCH ? ITEMS : 1];
         float ns = 0.0f;
-        {
+        if constexpr (PREFETCH) {
+            // request the next row of this slot now (nothing is fetched when there is none)
             const long nbase = nlive ? nrow * (long)cols : 0;
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
@@ -235,8 +235,21 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
                 buf_store<NW, kStream>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
             }
         }
+        if constexpr (PREFETCH) {
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+            for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+        } else {
+            // wide rows: no second copy of the row in registers; the next row is requested
+            // once this one is stored, and a second workgroup on the CU covers the wait
+            const long nbase = nlive ? nrow * (long)cols : 0;
+            const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
+            const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
+            if (nlive) ns = inv_rms[nrow];
+        }
         row = nrow; live = nlive; s = ns;
     }
 

@@ -343,6 +343,23 @@ def test_every_backward_workgroup_shape(block, tpr):
     U.assert_dw(dw, dw_ref)
 
 
+@pytest.mark.parametrize("prefetch", [0, 1])
+@pytest.mark.parametrize("cols", [1024, 16384])
+def test_backward_with_and_without_row_prefetch(prefetch, cols):
+    rows = 300
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=23)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "bf16")
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+    U.check(U.lib().mg_set_option(b"bwd_prefetch", prefetch))
+    try:
+        dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, "bf16")
+    finally:
+        U.check(U.lib().mg_set_option(b"bwd_prefetch", -1))
+    U.assert_matches(dx, dx_ref, "bf16", f"dx prefetch={prefetch}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+
+
 @pytest.mark.parametrize("tpr", [64, 128, 256, 512, 1024])
 def test_every_forward_workgroup_shape(tpr):
     rows, cols = 333, 4096
