@@ -135,6 +135,16 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
                   void* stream);
 
 /*
+ * Reports the launch shape mg_rmsnorm_fwd (backward == 0) or mg_rmsnorm_bwd (backward != 0)
+ * takes for rows of `cols` elements with 4-byte aligned base pointers; no counterpart in
+ * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
+ * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
+ * workgroup per row, *vectors_per_thread = 0).
+ */
+int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
+                           int* vectors_per_thread, int* workgroup_threads);
+
+/*
  * Measurement aid with no counterpart in the reference: a plain device-to-device copy of
  * `bytes` (a multiple of 16; both pointers 16-byte aligned) done by one kernel that moves
  * one 16-byte vector per thread.  Its HBM traffic is exactly 2*bytes, which makes it the

@@ -213,6 +213,25 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
     return MG_OK;
 }
 
+int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
+                            int* vectors_per_thread, int* workgroup_threads) {
+    int rc = check_rmsnorm_dims("mg_rmsnorm_launch_info", 1, cols, dtype);
+    if (rc != MG_OK) return rc;
+    if (generic == nullptr || threads_per_row == nullptr || vectors_per_thread == nullptr ||
+        workgroup_threads == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_launch_info: output pointers must not be NULL");
+    const int es = esize_of(dtype);
+    const long row_bytes = cols * es;
+    RowCfg cfg = {0, 0, 0, 0};
+    bool gen = opt_force_generic.load() != 0 || row_bytes % 4 != 0;
+    if (!gen) gen = backward ? !choose_bwd(row_bytes, es, &cfg) : !choose_fwd(row_bytes, &cfg);
+    *generic = gen ? 1 : 0;
+    *threads_per_row = gen ? 256 : cfg.tpr;
+    *vectors_per_thread = gen ? 0 : cfg.items;
+    *workgroup_threads = gen ? 256 : (backward ? cfg.block : (cfg.tpr > 256 ? cfg.tpr : 256));
+    return MG_OK;
+}
+
 int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num_partials, int64_t* ld) {
     int rc = check_rmsnorm_dims("mg_rmsnorm_bwd_workspace", rows, cols, dtype);
     if (rc != MG_OK) return rc;

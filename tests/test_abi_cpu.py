@@ -31,7 +31,8 @@ def _declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert _declared_functions() == sorted([
         "mg_abi_version", "mg_last_error", "mg_set_option", "mg_rmsnorm_fwd", "mg_rmsnorm_bwd_workspace",
-        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd", "mg_copy_bytes"])
+        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd", "mg_copy_bytes",
+        "mg_rmsnorm_launch_info"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -128,6 +129,41 @@ def test_copy_bytes_rejects_bad_arguments(lib):
     assert lib.mg_copy_bytes(FAKE, FAKE + 4, 32, None) == -1 and "aligned" in _err(lib)
     assert lib.mg_copy_bytes(None, FAKE, 32, None) == -1
     assert lib.mg_copy_bytes(None, None, 0, None) == 0
+
+
+def _launch_info(lib, backward, cols, dtype):
+    out = [ctypes.c_int(-1) for _ in range(4)]
+    assert lib.mg_rmsnorm_launch_info(backward, cols, dtype, *[ctypes.byref(o) for o in out]) == 0
+    return tuple(o.value for o in out)   # (generic, threads per row, vectors per thread, workgroup threads)
+
+
+@pytest.mark.parametrize("cols,dtype,fwd,bwd", [
+    # 2-byte types: 8 elements per 16-byte vector
+    (4096, 2, (0, 256, 2, 256), (0, 256, 2, 512)),      # metric shape: one row per 256-thread workgroup
+    (768, 2, (0, 64, 2, 256), (0, 64, 2, 512)),         # one wave per row
+    (2048, 1, (0, 128, 2, 256), (0, 128, 2, 512)),
+    (4100, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
+    (5120, 1, (0, 512, 2, 512), (0, 256, 3, 512)),
+    (8192, 2, (0, 512, 2, 512), (0, 512, 2, 512)),
+    (16384, 2, (0, 1024, 2, 1024), (0, 512, 4, 512)),
+    (4099, 2, (1, 256, 0, 256), (1, 256, 0, 256)),      # odd width of a 2-byte type: rows not 4-byte aligned
+    (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
+    # fp32: 4 elements per vector, any width is 4-byte aligned
+    (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
+    (33, 0, (0, 64, 1, 256), (0, 64, 1, 512)),
+    (16384, 0, (0, 1024, 4, 1024), (0, 512, 8, 512)),
+])
+def test_launch_shapes(lib, cols, dtype, fwd, bwd):
+    assert _launch_info(lib, 0, cols, dtype) == fwd
+    assert _launch_info(lib, 1, cols, dtype) == bwd
+
+
+def test_launch_info_rejects_bad_arguments(lib):
+    out = [ctypes.c_int() for _ in range(4)]
+    refs = [ctypes.byref(o) for o in out]
+    assert lib.mg_rmsnorm_launch_info(0, 0, 2, *refs) == -1
+    assert lib.mg_rmsnorm_launch_info(0, 128, 9, *refs) == -1
+    assert lib.mg_rmsnorm_launch_info(0, 128, 2, None, None, None, None) == -1
 
 
 def test_set_option(lib):
