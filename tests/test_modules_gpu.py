@@ -235,3 +235,59 @@ def test_module_forward_backward_under_graph_capture():
         assert torch.equal(out, want[0]), f"replay {i}: output"
         assert torch.equal(x.grad, want[1]), f"replay {i}: dx"
         assert torch.equal(norm.weight.grad, want[2]), f"replay {i}: dW"
+
+
+def test_concurrent_calls_from_several_threads():
+    """The library is re-entrant: four threads, each on its own stream, run forward+backward
+    at the same time and each gets the answer a lone call gives."""
+    import threading
+
+    from mgrrmsnorm_amd import ops
+
+    torch.manual_seed(11)
+    C = 2048
+    w = (1 + 0.02 * torch.randn(C, device="cuda")).to(torch.bfloat16)
+    xs = [torch.randn(300 + 17 * i, C, device="cuda").to(torch.bfloat16) for i in range(4)]
+    gs = [torch.randn_like(x) for x in xs]
+    want = []
+    for x, g in zip(xs, gs):
+        y, s = ops.rmsnorm_forward(x, w, 1e-6)
+        dx, dw32, _ = ops.rmsnorm_backward_f32(g, x, w, s)
+        want.append((y, dx, dw32))
+    torch.cuda.synchronize()
+    got, errors = [None] * 4, []
+
+    def work(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    y, s = ops.rmsnorm_forward(xs[i], w, 1e-6)
+                    dx, dw32, _ = ops.rmsnorm_backward_f32(gs[i], xs[i], w, s)
+            stream.synchronize()
+            got[i] = (y, dx, dw32)
+        except Exception as exc:  # surfaced below, in the main thread
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(4):
+        for a, b in zip(got[i], want[i]):
+            assert torch.equal(a, b), f"thread {i}"
+
+
+def test_double_backward_is_refused_cleanly():
+    """The backward pass is not itself differentiable (as in the reference, whose backward
+    calls an opaque extension): asking for a second derivative raises instead of returning
+    something wrong."""
+    from mgrrmsnorm_amd import RMSNorm
+
+    norm = RMSNorm(128).cuda()
+    x = torch.randn(4, 128, device="cuda", requires_grad=True)
+    (gx,) = torch.autograd.grad(norm(x).sum(), x, create_graph=True)
+    with pytest.raises(RuntimeError):
+        gx.sum().backward()
