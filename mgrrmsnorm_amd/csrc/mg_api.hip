@@ -127,15 +127,15 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
             if (bwd_cfg_ok(esize, tpr, need, b)) { *cfg = {kVec, tpr, need, b}; return true; }
     }
     for (int b : {block == 1024 ? 1024 : 512, 512}) {
-    for (int t = b; t >= 64; t /= 2) {
-        const int need = round_items(ceil_div(nvec, t));
-        const long in_flight = (long)(b / t) * row_bytes * 4;
-        if (in_flight >= 48 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
-    }
-    for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
-        const int need = round_items(ceil_div(nvec, t));
-        if (bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
-    }
+        for (int t = b; t >= 64; t /= 2) {
+            const int need = round_items(ceil_div(nvec, t));
+            const long in_flight = (long)(b / t) * row_bytes * 4;
+            if (in_flight >= 48 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+        }
+        for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
+            const int need = round_items(ceil_div(nvec, t));
+            if (bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+        }
     }
     return false;
 }
