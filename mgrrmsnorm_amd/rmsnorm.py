@@ -69,7 +69,17 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size))
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        return RMSNormFunction.apply(input, self.weight, self.epsilon)
+        weight = self.weight
+        if torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad):
+            return RMSNormFunction.apply(input, weight, self.epsilon)
+        # nothing to differentiate (inference, torch.no_grad()): same kernel, without the
+        # autograd node and its saved tensors
+        shape = input.shape
+        if len(shape) < 1:
+            raise RuntimeError("RMSNorm needs at least one dimension")
+        x2d = (input if input.is_contiguous() else input.contiguous()).view(-1, shape[-1])
+        w = weight if weight.is_contiguous() else weight.contiguous()
+        return ops.rmsnorm_forward(x2d, w, self.epsilon)[0].view(shape)
 
     def extra_repr(self) -> str:
         return f"hidden_size={self.hidden_size}, eps={self.epsilon}"

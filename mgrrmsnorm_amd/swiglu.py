@@ -61,7 +61,13 @@ class MegaGemmTriton(nn.Module):
         self.w3 = nn.Linear(self.hidden, d_model, bias=False)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.w3(MegaGemmFunction.apply(self.w12(x), self.hidden))
+        fused = self.w12(x)
+        if torch.is_grad_enabled() and fused.requires_grad:
+            return self.w3(MegaGemmFunction.apply(fused, self.hidden))
+        # nothing to differentiate: same kernel, without the autograd node
+        fused = fused if fused.is_contiguous() else fused.contiguous()
+        act = ops.swiglu_forward(fused.view(-1, 2 * self.hidden), self.hidden)
+        return self.w3(act.view(*fused.shape[:-1], self.hidden))
 
     def extra_repr(self) -> str:
         return f"d_model={self.w12.in_features}, hidden={self.hidden} (Triton Accelerated)"

@@ -291,3 +291,24 @@ def test_double_backward_is_refused_cleanly():
     (gx,) = torch.autograd.grad(norm(x).sum(), x, create_graph=True)
     with pytest.raises(RuntimeError):
         gx.sum().backward()
+
+
+def test_inference_path_equals_autograd_path():
+    """Under torch.no_grad() the modules skip the autograd node; outputs are bit-identical."""
+    from mgrrmsnorm_amd import MegaGemmTriton, RMSNorm
+
+    torch.manual_seed(4)
+    norm = RMSNorm(1024, 1e-6).cuda().to(torch.bfloat16)
+    mlp = MegaGemmTriton(1024).cuda().to(torch.bfloat16)
+    x = torch.randn(3, 50, 1024, device="cuda", dtype=torch.bfloat16)
+    y_grad = mlp(norm(x))
+    assert y_grad.requires_grad
+    with torch.no_grad():
+        y_inf = mlp(norm(x))
+    assert not y_inf.requires_grad and torch.equal(y_grad.detach(), y_inf)
+    for p in list(norm.parameters()) + list(mlp.parameters()):
+        p.requires_grad_(False)
+    assert torch.equal(mlp(norm(x)), y_inf)          # frozen weights, input without grad
+    xg = x.clone().requires_grad_(True)              # frozen weights, input with grad: autograd path
+    mlp(norm(xg)).sum().backward()
+    assert xg.grad is not None
