@@ -57,6 +57,7 @@ SHAPES = [
     (2, 20000),
     (3, 33000),      # wider than the register-resident kernels hold for 2-byte types
     (1000, 12),
+    (2, 65536),      # the widest row the forward register-resident kernels hold for 2-byte types
 ]
 
 
