@@ -230,6 +230,43 @@ def committed_traffic(kernel, workload):
         return None
 
 
+SWEEP = [
+    "rmsnorm_fwd_bwd_4096x4096_bf16", "rmsnorm_fwd_4096x4096_fp16", "rmsnorm_fwd_bwd_16384x8192_bf16",
+    "rmsnorm_fwd_bwd_65536x768_bf16", "rmsnorm_fwd_bwd_65536x2048_fp16", "rmsnorm_fwd_bwd_65536x4100_bf16",
+    "rmsnorm_fwd_bwd_65536x5120_fp16", "rmsnorm_fwd_bwd_65536x16384_bf16", "rmsnorm_fwd_bwd_16384x16384_fp32",
+    "swiglu_fwd_bwd_8192x11008_bf16",
+]
+
+
+def sweep(lib):
+    """Per-kernel and per-step figures for every benchmark configuration."""
+    import gc
+
+    rows = []
+    log(f"[sweep] {'workload':<36} " + " ".join(f"{k:>22}" for k in ("forward", "backward", "step")))
+    for name in SWEEP:
+        wl = make_workload(lib, name)
+        big = wl.step_bytes > 1e9
+        rec = {"workload": name}
+        cells = []
+        for kname, nbytes in wl.kernels.items():
+            t = time_kernel(wl, kname, launches=50 if big else 200)
+            rec[kname] = {"us": round(t * 1e6, 2), "GB/s": round(nbytes / t / 1e9, 1)}
+            cells.append(f"{t * 1e6:9.1f} us {nbytes / t / 1e9:6.0f} GB/s")
+        if len(cells) == 1:
+            cells.append(" " * 22)
+        steps = 20 if big else 100
+        ts = time_steps(wl, steps, 5, "eager") / steps
+        rec["step"] = {"us": round(ts * 1e6, 2), "GB/s": round(wl.step_bytes / ts / 1e9, 1)}
+        cells.append(f"{ts * 1e6:9.1f} us {wl.step_bytes / ts / 1e9:6.0f} GB/s")
+        log(f"[sweep] {name:<36} " + " ".join(cells))
+        rows.append(rec)
+        del wl
+        gc.collect()
+        torch.cuda.empty_cache()
+    return rows
+
+
 # -------------------------------------------------------------------------- CPU baseline
 
 def cpu_baseline(wl, budget_s=12.0):
@@ -283,6 +320,9 @@ def main():
     ap.add_argument("--launch", choices=["graph", "eager", "best"], default="best",
                     help="how the K timed steps are enqueued: one HIP graph, one by one, or the faster of the two")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sweep", action="store_true",
+                    help="additionally time every configuration of the hidden-size sweep, the large RMSNorm shape "
+                         "and the SwiGLU shape (per-kernel and per-step GB/s, table on stderr, 'sweep' in the JSON)")
     ap.add_argument("--calibrate-copies", type=int, default=0,
                     help="also launch this many plain copies of one activation tensor (mg_copy_bytes), so that a "
                          "counter profile of this run holds a kernel of known HBM traffic")
@@ -342,8 +382,11 @@ def main():
         "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
         "kernels": kern, "roofline": roofline,
     }
+    if args.sweep:
+        del wl
+        out["sweep"] = sweep(lib)
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl)
+        out["cpu_baseline"] = cpu_baseline(make_workload(lib, args.workload) if args.sweep else wl)
         log(f"[bench] cpu baseline: {out['cpu_baseline']}")
     print(json.dumps(out), flush=True)
 
