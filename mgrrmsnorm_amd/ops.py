@@ -87,9 +87,10 @@ def _bwd_workspace(lib, dev, rows, cols, code):
 
 
 def rmsnorm_backward_f32(grad_output: torch.Tensor, input: torch.Tensor, weight: torch.Tensor,
-                         inv_rms: torch.Tensor):
+                         inv_rms: torch.Tensor, need_weight_grad: bool = True):
     """Backward with dW kept in fp32: returns (grad_input, grad_weight_f32, grad_weight_cast)
-    where grad_weight_cast has the weight's dtype (it is grad_weight_f32 itself for fp32)."""
+    where grad_weight_cast has the weight's dtype (it is grad_weight_f32 itself for fp32).
+    With need_weight_grad=False the dW reduction is not launched and both are None."""
     if not (grad_output.is_cuda and input.is_cuda and weight.is_cuda and inv_rms.is_cuda
             and grad_output.is_contiguous() and input.is_contiguous() and weight.is_contiguous()
             and inv_rms.is_contiguous()):
@@ -112,17 +113,20 @@ def rmsnorm_backward_f32(grad_output: torch.Tensor, input: torch.Tensor, weight:
         n_part, ld = _bwd_workspace(lib, dev, rows, cols, code)
         grad_input = torch.empty_like(input)
         partial = torch.empty((n_part, ld), dtype=torch.float32, device=dev)
-        dw_f32 = torch.empty((cols,), dtype=torch.float32, device=dev)
-        dw_cast = dw_f32 if code == _lib.MG_F32 else torch.empty_like(weight)
+        dw_f32 = dw_cast = None
+        if need_weight_grad:
+            dw_f32 = torch.empty((cols,), dtype=torch.float32, device=dev)
+            dw_cast = dw_f32 if code == _lib.MG_F32 else torch.empty_like(weight)
         rc = lib.mg_rmsnorm_bwd(grad_input.data_ptr(), partial.data_ptr(), grad_output.data_ptr(),
                                 input.data_ptr(), weight.data_ptr(), inv_rms.data_ptr(), rows, cols, code,
                                 n_part, ld, stream)
         if rc != 0:
             _lib.check(rc, "RMSNorm backward")
-        rc = lib.mg_rmsnorm_dw_reduce(dw_f32.data_ptr(), None if dw_cast is dw_f32 else dw_cast.data_ptr(), code,
-                                      partial.data_ptr(), n_part, ld, cols, stream)
-        if rc != 0:
-            _lib.check(rc, "RMSNorm backward (dW reduction)")
+        if need_weight_grad:
+            rc = lib.mg_rmsnorm_dw_reduce(dw_f32.data_ptr(), None if dw_cast is dw_f32 else dw_cast.data_ptr(),
+                                          code, partial.data_ptr(), n_part, ld, cols, stream)
+            if rc != 0:
+                _lib.check(rc, "RMSNorm backward (dW reduction)")
     return grad_input, dw_f32, dw_cast
 
 

@@ -44,7 +44,7 @@ class RMSNormFunction(torch.autograd.Function):
         dy2d = (grad_output if grad_output.is_contiguous() else grad_output.contiguous()).view(x2d.shape)
         if dy2d.dtype != x2d.dtype:
             dy2d = dy2d.to(x2d.dtype)
-        dx2d, _, dw = ops.rmsnorm_backward_f32(dy2d, x2d, w, inv_rms)
+        dx2d, _, dw = ops.rmsnorm_backward_f32(dy2d, x2d, w, inv_rms, need_weight_grad=ctx.needs_input_grad[1])
         return dx2d.view(ctx.orig_shape), dw, None
 
 

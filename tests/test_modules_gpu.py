@@ -312,3 +312,18 @@ def test_inference_path_equals_autograd_path():
     xg = x.clone().requires_grad_(True)              # frozen weights, input with grad: autograd path
     mlp(norm(xg)).sum().backward()
     assert xg.grad is not None
+
+
+def test_frozen_weight_skips_the_dw_reduction():
+    from mgrrmsnorm_amd import RMSNorm
+
+    norm = RMSNorm(512, 1e-6).cuda()
+    x = torch.randn(40, 512, device="cuda", requires_grad=True)
+    norm(x).sum().backward()
+    want = x.grad.clone()
+    assert norm.weight.grad is not None
+    norm.weight.requires_grad_(False)
+    norm.weight.grad = None
+    x.grad = None
+    norm(x).sum().backward()
+    assert norm.weight.grad is None and torch.equal(x.grad, want)
