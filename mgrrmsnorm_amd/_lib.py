@@ -122,4 +122,8 @@ class device_of:
 
 
 def set_option(key: str, value: int) -> None:
+    """Tuning hook (mg_set_option); also drops the workspace shapes remembered by ops."""
     check(load().mg_set_option(key.encode(), int(value)), "mg_set_option")
+    from . import ops
+
+    ops._workspace_shapes.clear()

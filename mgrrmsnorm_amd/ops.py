@@ -70,6 +70,7 @@ def rmsnorm_forward(input: torch.Tensor, weight: torch.Tensor, epsilon: float):
 
 
 # (device index, rows, cols, dtype code) -> (num_partials, ld); the answer depends on nothing else
+# but the tuning options, and _lib.set_option() clears this table
 _workspace_shapes: dict = {}
 
 
