@@ -63,8 +63,8 @@ const char* mg_last_error(void);
  *
  * x, y: [rows, cols] of `dtype`; w: [cols] of the same dtype.  Any cols >= 1 is accepted
  * (the reference requires cols % 4 == 0 for fp32 and cols % 2 == 0 otherwise and skips a
- * remainder).  Base pointers must be aligned to the element size; the fast path is taken
- * when they are 4-byte aligned and cols*sizeof(element) is a multiple of 4.
+ * remainder).  Base pointers must be aligned to the element size; nothing more is needed
+ * for the fast path.
  * Limits: cols * sizeof(element) < 2^31, rows < 2^31.
  */
 int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w,
@@ -136,7 +136,7 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
 
 /*
  * Reports the launch shape mg_rmsnorm_fwd (backward == 0) or mg_rmsnorm_bwd (backward != 0)
- * takes for rows of `cols` elements with 4-byte aligned base pointers; no counterpart in
+ * takes for rows of `cols` elements; no counterpart in
  * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
  * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
  * workgroup per row, *vectors_per_thread = 0).

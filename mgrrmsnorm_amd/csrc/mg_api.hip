@@ -80,14 +80,10 @@ int cu_count(int* out) {
 
 int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }
 
-// The register-resident kernels need rows that start and end on 4-byte boundaries
-// (16-byte buffer accesses take any dword-aligned address and are range-checked per dword).
-bool rows_vectorizable(long row_bytes, std::initializer_list<const void*> ptrs) {
-    if (row_bytes % 4 != 0) return false;
-    for (const void* p : ptrs)
-        if (p != nullptr && !aligned(p, 4)) return false;
-    return true;
-}
+// The register-resident kernels take any row pitch and any element-aligned base: 16-byte
+// buffer accesses work at every byte alignment (measured at 2-, 4- and 8-byte offsets), the
+// range check is per dword, and the half dword that ends a row of an odd number of 2-byte
+// elements is handled by the lane that owns it.
 
 int round_items(int items) { return (items == 5 || items == 7) ? items + 1 : items; }
 
@@ -202,7 +198,7 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) generic = !rows_vectorizable(row_bytes, {y, x, w}) || !choose_fwd(row_bytes, &cfg);
+    if (!generic) generic = !choose_fwd(row_bytes, &cfg);
     const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps, xcd_group_or(kXcdGroupStreaming)};
     hipStream_t s = (hipStream_t)stream;
     hipError_t e = by_dtype(
@@ -223,7 +219,7 @@ int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, 
     const int es = esize_of(dtype);
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
-    bool gen = opt_force_generic.load() != 0 || row_bytes % 4 != 0;
+    bool gen = opt_force_generic.load() != 0;
     if (!gen) gen = backward ? !choose_bwd(row_bytes, es, &cfg) : !choose_fwd(row_bytes, &cfg);
     *generic = gen ? 1 : 0;
     *threads_per_row = gen ? 256 : cfg.tpr;
@@ -249,7 +245,7 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
     const int es = esize_of(dtype);
     RowCfg cfg = {0, 0, 0, 0};
     int rg = 1, dflt_per_cu = 1;
-    if (cols * es % 4 == 0 && opt_force_generic.load() == 0 && choose_bwd(cols * es, es, &cfg)) {
+    if (opt_force_generic.load() == 0 && choose_bwd(cols * es, es, &cfg)) {
         rg = cfg.block / cfg.tpr;
         dflt_per_cu = cfg.items >= 4 ? 4 : 1;
     }
@@ -291,7 +287,7 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) generic = !rows_vectorizable(row_bytes, {dx, dy, x, w}) || !choose_bwd(row_bytes, es, &cfg);
+    if (!generic) generic = !choose_bwd(row_bytes, es, &cfg);
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,

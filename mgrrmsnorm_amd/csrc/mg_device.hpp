@@ -68,6 +68,64 @@ __device__ __forceinline__ void buf_store(rsrc_t r, u32 byte_off, const Words<NW
 }
 
 // ---------------------------------------------------------------------------------
+// Rows of an odd number of 2-byte elements end in half a dword.  The per-dword range check
+// drops that last dword (it loads as 0 and its store is discarded), so the one lane whose
+// vector holds the last element fetches and stores it with 2-byte accesses and patches it
+// into the low half of the right word; the high half stays 0, i.e. an element of value 0
+// beyond the end of the row, which adds nothing to any sum.
+// ---------------------------------------------------------------------------------
+struct RowTail {
+    bool any;    // the row has such a half dword (uniform over the launch)
+    int lane;    // lane (within the row's TPR threads) that owns it
+    int item;    // which of that lane's vectors
+    int word;    // which 32-bit word of the vector
+    u32 off;     // byte offset of the element in the row
+};
+
+template <typename T, int TPR>
+__device__ __forceinline__ RowTail row_tail(int cols, u32 row_bytes) {
+    RowTail t = {false, 0, 0, 0, 0};
+    if constexpr (sizeof(T) == 2) {
+        t.any = (row_bytes & 3u) != 0;
+        const u32 vec = (u32)(cols - 1) / 8u;   // 8 two-byte elements per 16-byte vector
+        t.lane = (int)(vec % TPR);
+        t.item = (int)(vec / TPR);
+        t.word = (int)(((u32)(cols - 1) % 8u) / 2u);
+        t.off = row_bytes - 2u;
+    }
+    return t;
+}
+
+// All ITEMS vectors of one row for this lane (vector i of lane l is vector l + i*TPR of the
+// row), plus the half-dword tail if this lane owns it.
+template <int NW, int ITEMS, int TPR, int POLICY>
+__device__ __forceinline__ void load_row(Words<NW> (&v)[ITEMS], rsrc_t r, int lir, const RowTail& t) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) v[i] = buf_load<NW, POLICY>(r, (u32)(lir + i * TPR) * (NW * 4));
+    if (t.any && lir == t.lane) {
+        const u32 bits = __builtin_amdgcn_raw_buffer_load_b16(r, (int)t.off, 0, POLICY);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+            for (int j = 0; j < NW; ++j)
+                if (i == t.item && j == t.word) v[i].v[j] = bits;
+    }
+}
+
+// Store vector `i` of this lane; the owner of the half-dword tail also stores that element.
+template <int NW, int TPR, int POLICY>
+__device__ __forceinline__ void store_item(rsrc_t r, int lir, int i, const Words<NW>& w, const RowTail& t) {
+    buf_store<NW, POLICY>(r, (u32)(lir + i * TPR) * (NW * 4), w);
+    if (t.any && lir == t.lane && i == t.item) {
+        u32 bits = 0;
+#pragma unroll
+        for (int j = 0; j < NW; ++j)
+            if (j == t.word) bits = w.v[j];
+        __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(bits & 0xffffu), r, (int)t.off, 0, POLICY);
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // Element traits: PER_WORD elements per 32-bit word, conversion to/from fp32.
 // fp32 -> fp16/bf16 uses the hardware round-to-nearest-even converts
 // (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32); never the round-toward-zero pack.

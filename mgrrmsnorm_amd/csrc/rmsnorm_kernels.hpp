@@ -5,14 +5,14 @@
 // and each holds ITEMS vectors of it in VGPRs, vector i of thread t being vector t + i*TPR
 // of the row.  All of a row's loads are issued before the first use.  Row sums are reduced
 // with DPP inside a wave and through a few floats of LDS across the waves of a row.
-// Rows only need 4-byte alignment: buffer_load/store_dwordx4 take any dword-aligned
-// address, and the range check against the row's byte length is made per dword, so a row
-// whose length is not a multiple of 16 simply ends inside its last vector (the lanes and
-// dwords beyond it load 0 and store nothing).
+// Rows need no alignment beyond that of an element: buffer_load/store_dwordx4 work at any
+// byte offset, and the range check against the row's byte length is made per dword, so a
+// row whose length is not a multiple of 16 simply ends inside its last vector (the lanes
+// and dwords beyond it load 0 and store nothing).  A row of an odd number of 2-byte
+// elements ends in half a dword, which one lane moves with 2-byte accesses (RowTail).
 //
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
-// the row; used when the row pitch or a base pointer is not a multiple of 4 bytes, or the
-// row does not fit the register-resident family.
+// the row; used when the row does not fit the register-resident family (or on request).
 #pragma once
 #include "mg_device.hpp"
 
@@ -45,12 +45,11 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
     const rsrc_t ry = make_rsrc(y + base, live ? row_bytes : 0u);
     const rsrc_t rw = make_rsrc(w, row_bytes);
 
+    const RowTail tail = row_tail<T, TPR>(cols, row_bytes);
     Words<NW> xv[ITEMS];
     Words<NW> wv[ITEMS];
-#pragma unroll
-    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
-#pragma unroll
-    for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW>(rw, (u32)(lir + i * TPR) * VEC);
+    load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
+    load_row<NW, ITEMS, TPR, kKeep>(wv, rw, lir, tail);
 
     float ss = 0.0f;
 #pragma unroll
@@ -81,7 +80,7 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
         unpack_vec<T, NW>(wv[i], wf);
 #pragma unroll
         for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
-        buf_store<NW, kStream>(ry, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+        store_item<NW, TPR, kStream>(ry, lir, i, pack_vec<T, NW>(o), tail);
     }
 }
 
@@ -154,12 +153,9 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
 #pragma unroll
         for (int k = 0; k < EPV; ++k) acc[i][k] = 0.0f;
 
+    const RowTail tail = row_tail<T, TPR>(cols, row_bytes);
     Words<NW> wv[ITEMS];
-    {
-        const rsrc_t rw = make_rsrc(w, row_bytes);
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW>(rw, (u32)(lir + i * TPR) * VEC);
-    }
+    load_row<NW, ITEMS, TPR, kKeep>(wv, make_rsrc(w, row_bytes), lir, tail);
 
     Words<NW> xv[ITEMS], gv[ITEMS];
     long row = slot;
@@ -169,10 +165,8 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
         const long base = live ? row * (long)cols : 0;
         const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
         const rsrc_t rg_ = make_rsrc(dy + base, live ? row_bytes : 0u);
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
-#pragma unroll
-        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
+        load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
+        load_row<NW, ITEMS, TPR, kStream>(gv, rg_, lir, tail);
         if (live) s = inv_rms[row];
     }
 
@@ -186,10 +180,8 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
             const long nbase = nlive ? nrow * (long)cols : 0;
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
+            load_row<NW, ITEMS, TPR, kStream>(nxv, rx, lir, tail);
+            load_row<NW, ITEMS, TPR, kStream>(ngv, rg_, lir, tail);
             if (nlive) ns = inv_rms[nrow];
         }
 
@@ -232,7 +224,7 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
                 unpack_vec<T, NW>(wv[i], wf);
 #pragma unroll
                 for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
-                buf_store<NW, kStream>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
+                store_item<NW, TPR, kStream>(rd, lir, i, pack_vec<T, NW>(o), tail);
             }
         }
         if constexpr (PREFETCH) {
@@ -244,10 +236,8 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
             const long nbase = nlive ? nrow * (long)cols : 0;
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, (u32)(lir + i * TPR) * VEC);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<NW, kStream>(rg_, (u32)(lir + i * TPR) * VEC);
+            load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
+            load_row<NW, ITEMS, TPR, kStream>(gv, rg_, lir, tail);
             if (nlive) ns = inv_rms[nrow];
         }
         row = nrow; live = nlive; s = ns;

@@ -146,7 +146,7 @@ def _launch_info(lib, backward, cols, dtype):
     (5120, 1, (0, 512, 2, 512), (0, 256, 3, 512)),
     (8192, 2, (0, 512, 2, 512), (0, 512, 2, 512)),
     (16384, 2, (0, 1024, 2, 1024), (0, 512, 4, 512)),
-    (4099, 2, (1, 256, 0, 256), (1, 256, 0, 256)),      # odd width of a 2-byte type: rows not 4-byte aligned
+    (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
     # fp32: 4 elements per vector, any width is 4-byte aligned
     (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),

@@ -51,7 +51,9 @@ SHAPES = [
     (65, 5120),
     (33, 16384),
     (7, 100),
-    (5, 33),         # odd width: element-wise kernels for 2-byte types, vector kernels for fp32
+    (5, 33),         # odd width: rows of 2-byte types end in half a dword
+    (9, 4099),
+    (4, 8191),
     (3, 1),
     (1, 8),
     (2, 20000),
@@ -96,8 +98,8 @@ def test_outlier_rows(dtype, cols):
 
 @pytest.mark.parametrize("dtype", ALL)
 def test_generic_kernels_match_oracle(dtype):
-    """The element-wise path forced on an aligned shape, and taken naturally for a base
-    pointer that is not 16-byte aligned."""
+    """The element-wise path forced on a shape the vector kernels would take; then the vector
+    kernels on a base pointer that is aligned to the element size only."""
     rows, cols = 100, 1024
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=99)
     y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
