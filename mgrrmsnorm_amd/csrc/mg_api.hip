@@ -93,6 +93,10 @@ int round_items(int items) { return (items == 5 || items == 7) ? items + 1 : ite
 bool choose_fwd(long row_bytes, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
+    {   // rows narrower than a wave: several rows per wave (a requested 8 or 16 wins when it fits)
+        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes) : 0);
+        if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 0}; return true; }
+    }
     if (tpr_ok(tpr)) {
         const int need = ceil_div(nvec, tpr) == 7 ? 8 : ceil_div(nvec, tpr);
         if (need <= kFwdMaxItems && fwd_items_ok(need)) { *cfg = {kVec, tpr, need, 0}; return true; }
@@ -117,6 +121,10 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
 bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
+    {   // rows narrower than a wave: several rows per wave, always 512-thread workgroups
+        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes) : 0);
+        if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 512}; return true; }
+    }
     if (tpr_ok(tpr)) {
         const int need = round_items(ceil_div(nvec, tpr));
         for (int b : {block, 512, 1024})
@@ -248,6 +256,8 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
     if (opt_force_generic.load() == 0 && choose_bwd(cols * es, es, &cfg)) {
         rg = cfg.block / cfg.tpr;
         dflt_per_cu = cfg.items >= 4 ? 4 : 1;
+        // one vector per lane leaves half the bytes in flight: a second workgroup makes up for it
+        if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;

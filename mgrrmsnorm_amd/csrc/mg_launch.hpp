@@ -9,7 +9,7 @@ namespace mg {
 // How a row is spread over threads in the register-resident RMSNorm kernels.
 struct RowCfg {
     int vec;    // bytes per vector load (16)
-    int tpr;    // threads per row: 64, 128, 256, 512, 1024
+    int tpr;    // threads per row: 64, 128, 256, 512, 1024; 8 or 16 = several rows per wave
     int items;  // vectors per thread
     int block;  // backward only: threads per workgroup, 1024 or 512
 };
@@ -32,6 +32,19 @@ constexpr bool bwd_cfg_ok(int esize, int tpr, int items, int block) {
            (tpr == block || tpr * items * (kVec / esize) * 4 <= 65536);
 }
 constexpr bool tpr_ok(int tpr) { return tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024; }
+
+// Rows of at most 64 vectors whose pitch is a multiple of 16 bytes can share a wave:
+// 8 or 16 lanes per row, 1, 2 or 4 vectors per lane.
+constexpr bool narrow_tpr(int tpr) { return tpr == 8 || tpr == 16; }
+constexpr int narrow_items(long row_bytes, int tpr) {   // 0 = does not fit
+    if (!narrow_tpr(tpr) || row_bytes % kVec != 0) return 0;
+    const long need = (row_bytes / kVec + tpr - 1) / tpr;
+    return need <= 2 ? (int)need : (need <= 4 ? 4 : 0);
+}
+// Default use: rows of up to 32 vectors (512 bytes); wider rows fill a wave on their own.
+constexpr int narrow_default_tpr(long row_bytes) {
+    return (row_bytes % kVec != 0 || row_bytes > 512) ? 0 : (row_bytes <= 256 ? 8 : 16);
+}
 
 struct FwdArgs {
     void* y; float* inv_rms; const void* x; const void* w;

@@ -45,6 +45,25 @@ hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
     }
 }
 
+template <int TPR, int ITEMS>
+hipError_t run_narrow(const BwdArgs& a, hipStream_t s) {
+    rmsnorm_bwd_narrow<elem_t, TPR, ITEMS><<<dim3((unsigned)a.num_partials), dim3(512), 0, s>>>(
+        (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+        a.rows, a.cols, 1.0f / (float)a.cols);
+    return hipGetLastError();
+}
+
+template <int TPR>
+hipError_t narrow_by_items(int items, const BwdArgs& a, hipStream_t s) {
+    if (narrow_items((long)a.cols * (long)sizeof(elem_t), TPR) != items) return hipErrorInvalidValue;
+    switch (items) {
+        case 1: return run_narrow<TPR, 1>(a, s);
+        case 2: return run_narrow<TPR, 2>(a, s);
+        case 4: return run_narrow<TPR, 4>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 template <int BLOCK>
 hipError_t by_tpr(int tpr, int items, const BwdArgs& a, hipStream_t s) {
     switch (tpr) {
@@ -75,6 +94,8 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
         return hipGetLastError();
     }
     if (cfg.vec != kVec) return hipErrorInvalidValue;
+    if (cfg.tpr == 8 && cfg.block == 512) return narrow_by_items<8>(cfg.items, a, s);
+    if (cfg.tpr == 16 && cfg.block == 512) return narrow_by_items<16>(cfg.items, a, s);
     if (cfg.block == 1024) return by_tpr<1024>(cfg.tpr, cfg.items, a, s);
     if (cfg.block == 512) return by_tpr<512>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;

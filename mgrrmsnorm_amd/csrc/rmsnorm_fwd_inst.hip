@@ -43,9 +43,32 @@ hipError_t by_items(int items, const FwdArgs& a, hipStream_t s) {
     }
 }
 
+template <int TPR, int ITEMS>
+hipError_t run_narrow(const FwdArgs& a, hipStream_t s) {
+    constexpr int RPB = 256 / TPR;
+    const long grid = (a.rows + RPB - 1) / RPB;
+    rmsnorm_fwd_narrow<elem_t, TPR, ITEMS><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
+        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+        1.0f / (float)a.cols, a.xcd_group);
+    return hipGetLastError();
+}
+
+template <int TPR>
+hipError_t narrow_by_items(int items, const FwdArgs& a, hipStream_t s) {
+    if (narrow_items((long)a.cols * (long)sizeof(elem_t), TPR) != items) return hipErrorInvalidValue;
+    switch (items) {
+        case 1: return run_narrow<TPR, 1>(a, s);
+        case 2: return run_narrow<TPR, 2>(a, s);
+        case 4: return run_narrow<TPR, 4>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 template <int VEC>
 hipError_t by_tpr(int tpr, int items, const FwdArgs& a, hipStream_t s) {
     switch (tpr) {
+        case 8: return narrow_by_items<8>(items, a, s);
+        case 16: return narrow_by_items<16>(items, a, s);
         case 64: return by_items<VEC, 64>(items, a, s);
         case 128: return by_items<VEC, 128>(items, a, s);
         case 256: return by_items<VEC, 256>(items, a, s);

@@ -85,6 +85,218 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
 }
 
 // =================================================================================
+// Narrow rows (at most 32 vectors, row pitch a multiple of 16 bytes): TPR = 8 or 16 lanes per
+// row, so a wave carries 64/TPR consecutive rows and a 256-thread workgroup 256/TPR.  One
+// buffer resource spans the wave's rows; lanes past the end of a row, and rows past the end
+// of the matrix, get an out-of-range offset (loads 0, stores nothing).  Row sums stay inside
+// the 16-lane DPP rows: no LDS, no barrier.
+// =================================================================================
+constexpr u32 kOutOfRange = 0xFFFFFFF0u;
+
+template <typename T, int TPR, int ITEMS>
+__global__ void __launch_bounds__(256)
+rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                   const T* __restrict__ w, long rows, int cols, float eps, float inv_cols, int xcd_group) {
+    constexpr int RPW = kWave / TPR;   // rows per wave
+    constexpr int RPB = 256 / TPR;     // rows per workgroup
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int lane = tid & (kWave - 1);
+    const int sub = lane / TPR;        // row inside the wave
+    const int lir = lane % TPR;        // lane inside the row
+    const long row0 = xcd_remap(blockIdx.x, gridDim.x, xcd_group) * RPB + (long)wave * RPW;
+    const long left = rows - row0;
+    const u32 live_rows = left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = row_bytes / 16u;
+    const long base = live_rows ? row0 * (long)cols : 0;
+    const rsrc_t rx = make_rsrc(x + base, live_rows * row_bytes);
+    const rsrc_t ry = make_rsrc(y + base, live_rows * row_bytes);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+
+    Words<4> xv[ITEMS], wv[ITEMS];
+    u32 off[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const u32 vec = (u32)(lir + i * TPR);
+        off[i] = vec < nvec ? (u32)sub * row_bytes + vec * 16u : kOutOfRange;
+        xv[i] = buf_load<4, kStream>(rx, off[i]);
+        wv[i] = buf_load<4, kKeep>(rw, vec < nvec ? vec * 16u : kOutOfRange);
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float f[EPV];
+        unpack_vec<T, 4>(xv[i], f);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) ss = __builtin_fmaf(f[k], f[k], ss);
+    }
+    ss = group_sum<TPR>(ss);
+    const float s = fast_rsqrt(ss * inv_cols + eps);
+    if (lir == 0 && (u32)sub < live_rows && inv_rms != nullptr) inv_rms[row0 + sub] = s;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float xf[EPV], wf[EPV], o[EPV];
+        unpack_vec<T, 4>(xv[i], xf);
+        unpack_vec<T, 4>(wv[i], wf);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
+        buf_store<4, kStream>(ry, off[i], pack_vec<T, 4>(o));
+    }
+}
+
+// Backward pass 1 for narrow rows: persistent grid of 512-thread workgroups; each wave walks
+// groups of 64/TPR consecutive rows (group g of wave q: rows (g*Q + q)*RPW ..., Q = all waves),
+// prefetching the next group.  dW: per lane in registers, then across the rows of a wave by
+// lane shuffles, then across the 8 waves in wave order through LDS; one partial row per
+// workgroup.
+template <typename T, int TPR, int ITEMS>
+__global__ void __launch_bounds__(512)
+rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
+                   const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
+                   long rows, int cols, float inv_cols) {
+    constexpr int BLOCK = 512;
+    constexpr int WAVES = BLOCK / kWave;
+    constexpr int RPW = kWave / TPR;
+    constexpr int EPV = 16 / (int)sizeof(T);
+    constexpr int COVER = TPR * ITEMS * EPV;   // columns one row's lanes cover (>= cols)
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int lane = tid & (kWave - 1);
+    const int sub = lane / TPR;
+    const int lir = lane % TPR;
+    const long nwaves = (long)gridDim.x * WAVES;
+    const long q = (long)blockIdx.x * WAVES + wave;
+    const long ngroups = (rows + RPW - 1) / RPW;            // groups of RPW rows in the matrix
+    const long n_it = (ngroups + nwaves - 1) / nwaves;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = row_bytes / 16u;
+
+    float acc[ITEMS][EPV];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) acc[i][k] = 0.0f;
+
+    Words<4> wv[ITEMS];
+    u32 voff[ITEMS];   // offset inside the wave's rows, or out of range
+    {
+        const rsrc_t rw = make_rsrc(w, row_bytes);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            const u32 vec = (u32)(lir + i * TPR);
+            voff[i] = vec < nvec ? (u32)sub * row_bytes + vec * 16u : kOutOfRange;
+            wv[i] = buf_load<4, kKeep>(rw, vec < nvec ? vec * 16u : kOutOfRange);
+        }
+    }
+
+    auto live_rows_of = [&](long row0) -> u32 {
+        const long left = rows - row0;
+        return left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
+    };
+
+    Words<4> xv[ITEMS], gv[ITEMS];
+    long row0 = q * RPW;
+    u32 live = live_rows_of(row0);
+    float s = 0.0f;
+    {
+        const long base = live ? row0 * (long)cols : 0;
+        const rsrc_t rx = make_rsrc(x + base, live * row_bytes);
+        const rsrc_t rg = make_rsrc(dy + base, live * row_bytes);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<4, kStream>(rx, voff[i]);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<4, kStream>(rg, voff[i]);
+        if ((u32)sub < live) s = inv_rms[row0 + sub];
+    }
+
+    for (long it = 0; it < n_it; ++it) {
+        const long nrow0 = row0 + nwaves * RPW;
+        const u32 nlive = live_rows_of(nrow0);
+        Words<4> nxv[ITEMS], ngv[ITEMS];
+        float ns = 0.0f;
+        {
+            const long nbase = nlive ? nrow0 * (long)cols : 0;
+            const rsrc_t rx = make_rsrc(x + nbase, nlive * row_bytes);
+            const rsrc_t rg = make_rsrc(dy + nbase, nlive * row_bytes);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<4, kStream>(rx, voff[i]);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<4, kStream>(rg, voff[i]);
+            if ((u32)sub < nlive) ns = inv_rms[nrow0 + sub];
+        }
+
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            float xf[EPV], gf[EPV], wf[EPV];
+            unpack_vec<T, 4>(xv[i], xf);
+            unpack_vec<T, 4>(gv[i], gf);
+            unpack_vec<T, 4>(wv[i], wf);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                const float t = gf[k] * xf[k];
+                a = __builtin_fmaf(t, wf[k], a);
+                acc[i][k] = __builtin_fmaf(t, s, acc[i][k]);
+            }
+        }
+        a = group_sum<TPR>(a);
+        const float c2 = a * (s * s) * s * inv_cols;
+        {
+            const long base = live ? row0 * (long)cols : 0;
+            const rsrc_t rd = make_rsrc(dx + base, live * row_bytes);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                float xf[EPV], gf[EPV], wf[EPV], o[EPV];
+                unpack_vec<T, 4>(xv[i], xf);
+                unpack_vec<T, 4>(gv[i], gf);
+                unpack_vec<T, 4>(wv[i], wf);
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
+                buf_store<4, kStream>(rd, voff[i], pack_vec<T, 4>(o));
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+        row0 = nrow0; live = nlive; s = ns;
+    }
+
+    // rows of one wave: lanes lir, lir + TPR, lir + 2*TPR, ... hold the same columns
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+        for (int k = 0; k < EPV; ++k)
+#pragma unroll
+            for (int d = TPR; d < kWave; d *= 2) acc[i][k] += __shfl_xor(acc[i][k], d);
+
+    // waves of the workgroup, in wave order
+    __shared__ float dwbuf[COVER];
+    for (int g = 0; g < WAVES; ++g) {
+        if (wave == g && sub == 0) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                const int c0 = (lir + i * TPR) * EPV;
+#pragma unroll
+                for (int k = 0; k < EPV; ++k) {
+                    if (g == 0) dwbuf[c0 + k] = acc[i][k];
+                    else dwbuf[c0 + k] += acc[i][k];
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float* out = dw_part + (long)blockIdx.x * ld;
+    const int lim = ld < COVER ? ld : COVER;
+    for (int c = tid * 4; c < lim; c += BLOCK * 4) {
+        f32x4 v = {dwbuf[c], dwbuf[c + 1], dwbuf[c + 2], dwbuf[c + 3]};
+        *reinterpret_cast<f32x4*>(out + c) = v;
+    }
+    // columns between COVER and ld (COVER can be as small as 32) belong to no lane
+    for (int c = COVER + tid; c < ld; c += BLOCK) out[c] = 0.0f;
+}
+
+// =================================================================================
 // Forward, generic: one workgroup of 256 threads per row, any cols, any alignment.
 // =================================================================================
 template <typename T>

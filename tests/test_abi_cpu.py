@@ -148,6 +148,14 @@ def _launch_info(lib, backward, cols, dtype):
     (16384, 2, (0, 1024, 2, 1024), (0, 512, 4, 512)),
     (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
+    # rows narrower than a wave whose pitch is a multiple of 16 bytes: 8 or 16 lanes per row
+    (64, 2, (0, 8, 1, 256), (0, 8, 1, 512)),            # 8 vectors: 8 rows per wave
+    (128, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # head-dimension 128
+    (256, 1, (0, 16, 2, 256), (0, 16, 2, 512)),
+    (8, 2, (0, 8, 1, 256), (0, 8, 1, 512)),             # a single vector per row
+    (264, 2, (0, 64, 1, 256), (0, 64, 1, 512)),         # 33 vectors: one wave per row again
+    (100, 2, (0, 64, 1, 256), (0, 64, 1, 512)),         # pitch 200 bytes: not a multiple of 16
+    (64, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
     # fp32: 4 elements per vector, any width is 4-byte aligned
     (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
     (33, 0, (0, 64, 1, 256), (0, 64, 1, 512)),

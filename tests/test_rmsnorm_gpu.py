@@ -60,6 +60,15 @@ SHAPES = [
     (3, 33000),      # wider than the register-resident kernels hold for 2-byte types
     (1000, 12),
     (2, 65536),      # the widest row the forward register-resident kernels hold for 2-byte types
+    # rows narrower than a wave (pitch a multiple of 16 bytes): several rows share a wave
+    (1000, 64),      # 8 lanes per row for 2-byte types; 1000 = 125 full waves of 8 rows
+    (1003, 128),     # the last wave holds 3 rows of its 8
+    (517, 256),      # 16 lanes per row, 2 vectors per lane
+    (259, 8),        # one vector per row (2-byte types), two for fp32
+    (37, 72),        # 9 vectors: the second vector of a lane exists for one lane only
+    (5000, 200),     # 25 vectors over 16 lanes
+    (3, 32),
+    (70000, 16),     # more rows than the backward grid has row slots at once
 ]
 
 
@@ -361,6 +370,30 @@ def test_backward_with_and_without_row_prefetch(prefetch, cols):
         U.check(U.lib().mg_set_option(b"bwd_prefetch", -1))
     U.assert_matches(dx, dx_ref, "bf16", f"dx prefetch={prefetch}", floor=floor)
     U.assert_dw(dw, dw_ref)
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("tpr", [8, 16])
+@pytest.mark.parametrize("cols", [32, 64, 128, 256])
+def test_every_narrow_row_shape(dtype, tpr, cols):
+    """8 and 16 lanes per row with 1, 2 and 4 vectors per lane, whichever the automatic choice
+    takes; a shape that does not fit the request falls back to the automatic one."""
+    rows = 333
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=31 + cols)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    L = U.lib()
+    U.check(L.mg_set_option(b"fwd_tpr", tpr)); U.check(L.mg_set_option(b"bwd_tpr", tpr))
+    try:
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+        dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    finally:
+        U.check(L.mg_set_option(b"fwd_tpr", 0)); U.check(L.mg_set_option(b"bwd_tpr", 0))
+    U.assert_matches(y, y_ref, dtype, f"y tpr={tpr}")
+    np.testing.assert_allclose(s.cpu().numpy(), s_ref, rtol=1e-6)
+    U.assert_matches(dx, dx_ref, dtype, f"dx tpr={tpr}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    assert torch.isfinite(part).all(), "padding columns of a partial row were left unwritten"
 
 
 @pytest.mark.parametrize("tpr", [64, 128, 256, 512, 1024])
