@@ -234,6 +234,9 @@ SWEEP = [
     "rmsnorm_fwd_bwd_4096x4096_bf16", "rmsnorm_fwd_4096x4096_fp16", "rmsnorm_fwd_bwd_16384x8192_bf16",
     "rmsnorm_fwd_bwd_65536x768_bf16", "rmsnorm_fwd_bwd_65536x2048_fp16", "rmsnorm_fwd_bwd_65536x4100_bf16",
     "rmsnorm_fwd_bwd_65536x5120_fp16", "rmsnorm_fwd_bwd_65536x16384_bf16", "rmsnorm_fwd_bwd_16384x16384_fp32",
+    # rows narrower than a wave (per-head QK-norm widths): several rows per wave
+    "rmsnorm_fwd_bwd_2097152x64_bf16", "rmsnorm_fwd_bwd_1048576x128_bf16", "rmsnorm_fwd_bwd_524288x256_bf16",
+    "rmsnorm_fwd_bwd_1048576x64_fp32",
     "swiglu_fwd_bwd_8192x11008_bf16",
 ]
 
