@@ -11,6 +11,9 @@
 // and dwords beyond it load 0 and store nothing).  A row of an odd number of 2-byte
 // elements ends in half a dword, which one lane moves with 2-byte accesses (RowTail).
 //
+// Narrow family: rows of at most 64 vectors whose pitch is a multiple of 16 bytes put 8 or
+// 16 lanes on a row, so that one wave carries 8 or 4 consecutive rows (see below).
+//
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
 // the row; used when the row does not fit the register-resident family (or on request).
 #pragma once
