@@ -48,14 +48,14 @@ def log(*a):
 class RmsNormWorkload:
     """fwd (+ bwd + dW reduce) on [rows, cols]; inputs N(0,1), w = 1 + 0.02 N(0,1), eps 1e-6."""
 
-    def __init__(self, lib, rows, cols, dtype, backward=True, seed=42):
+    def __init__(self, lib, rows, cols, dtype, backward=True, seed=42, nsets=0):
         self.lib, self.rows, self.cols, self.dtype, self.backward = lib, rows, cols, dtype, backward
         e = ESIZE[dtype]
         self.fwd_bytes = 2 * rows * cols * e + cols * e
         self.bwd_bytes = 3 * rows * cols * e + cols * e + 4 * cols
         self.step_bytes = self.fwd_bytes + (self.bwd_bytes if backward else 0)
         per_set = (4 if backward else 2) * rows * cols * e
-        self.nsets = max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
+        self.nsets = nsets if nsets > 0 else max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
         td = TORCH[dtype]
         g = torch.Generator(device="cuda").manual_seed(seed)
         self.w = (1 + 0.02 * torch.randn(cols, generator=g, device="cuda")).to(td)
@@ -114,13 +114,13 @@ class RmsNormWorkload:
 class SwigluWorkload:
     """Activation fwd + bwd on gu [M, 2H] (N(0,1)) and dh [M, H]."""
 
-    def __init__(self, lib, M, H, dtype, seed=42):
+    def __init__(self, lib, M, H, dtype, seed=42, nsets=0):
         self.lib, self.M, self.H, self.dtype = lib, M, H, dtype
         e = ESIZE[dtype]
         self.fwd_bytes, self.bwd_bytes = 3 * M * H * e, 5 * M * H * e
         self.step_bytes = self.fwd_bytes + self.bwd_bytes
         per_set = 6 * M * H * e
-        self.nsets = max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
+        self.nsets = nsets if nsets > 0 else max(2, -(-4 * INFINITY_CACHE_BYTES // per_set))
         td = TORCH[dtype]
         g = torch.Generator(device="cuda").manual_seed(seed)
         self.sets = []
@@ -156,13 +156,13 @@ class SwigluWorkload:
         return {"swiglu_fwd": self.fwd, "swiglu_bwd": self.bwd}[name]
 
 
-def make_workload(lib, name):
+def make_workload(lib, name, nsets=0):
     m = re.fullmatch(r"rmsnorm_(fwd_bwd|fwd)_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
     if m:
-        return RmsNormWorkload(lib, int(m.group(2)), int(m.group(3)), m.group(4), backward=m.group(1) == "fwd_bwd")
+        return RmsNormWorkload(lib, int(m.group(2)), int(m.group(3)), m.group(4), backward=m.group(1) == "fwd_bwd", nsets=nsets)
     m = re.fullmatch(r"swiglu_fwd_bwd_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
     if m:
-        return SwigluWorkload(lib, int(m.group(1)), int(m.group(2)), m.group(3))
+        return SwigluWorkload(lib, int(m.group(1)), int(m.group(2)), m.group(3), nsets=nsets)
     raise SystemExit(f"unknown workload '{name}'")
 
 
@@ -322,6 +322,9 @@ def main():
     ap.add_argument("--workload", default="rmsnorm_fwd_bwd_4096x4096_bf16")
     ap.add_argument("--launch", choices=["graph", "eager", "best"], default="best",
                     help="how the K timed steps are enqueued: one HIP graph, one by one, or the faster of the two")
+    ap.add_argument("--buffer-sets", type=int, default=0,
+                    help="input/output buffer sets the steps rotate over; 0 = enough to exceed four times the "
+                         "256 MiB Infinity Cache (the reported configuration), 1 = everything stays cache resident")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sweep", action="store_true",
                     help="additionally time every configuration of the hidden-size sweep, the large RMSNorm shape "
@@ -340,7 +343,7 @@ def main():
     from mgrrmsnorm_amd import _lib
     lib = _lib.load()
     torch.cuda.set_device(0)
-    wl = make_workload(lib, args.workload)
+    wl = make_workload(lib, args.workload, args.buffer_sets)
     log(f"[bench] {wl.name}: {wl.step_bytes / 1e6:.1f} MB algorithmic per step, {wl.nsets} buffer sets, "
         f"device {torch.cuda.get_device_name(0)}")
 
