@@ -170,7 +170,8 @@ def test_zero_input_rows_give_zero_output_and_scaled_gradient():
 
 # --------------------------------------------------------------------------- determinism
 
-@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 2000, 5120), ("fp32", 777, 1000)])
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 2000, 5120), ("fp32", 777, 1000),
+                                             ("bf16", 100003, 128), ("fp32", 50001, 64)])
 def test_dw_is_bit_identical_across_runs(dtype, rows, cols):
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=3)
     xd, dyd, wd = _dev(x, dy, w)
@@ -185,9 +186,9 @@ def test_dw_is_bit_identical_across_runs(dtype, rows, cols):
             assert torch.equal(first[0], dx)
 
 
+@pytest.mark.parametrize("rows,cols", [(515, 2048), (5003, 128)])
 @pytest.mark.parametrize("P", [1, 3, 64, 1000])
-def test_any_number_of_partials_gives_the_same_gradient(P):
-    rows, cols = 515, 2048
+def test_any_number_of_partials_gives_the_same_gradient(P, rows, cols):
     x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=11)
     _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "bf16")
     xd, dyd, wd = _dev(x, dy, w)
@@ -212,6 +213,8 @@ FULL = [
     ("fp16", 65536, 5120),
     ("bf16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
     ("fp32", 70000, 16388),   # 4.6 GB per tensor, rows 4-byte aligned only: offsets beyond 2^32
+    ("bf16", 2097152, 128),   # rows narrower than a wave: 8 rows per wave, 262144 waves
+    ("fp16", 1048576, 256),
 ]
 
 
@@ -237,7 +240,7 @@ def test_full_size_by_row_replication(dtype, rows, cols):
 
 
 @pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("bf16", 16384, 8192), ("bf16", 65536, 768),
-                                             ("fp32", 4096, 4096)])
+                                             ("fp32", 4096, 4096), ("bf16", 1048576, 64)])
 def test_power_of_two_scaling_is_exact(dtype, rows, cols):
     """Scaling dy (or w in the forward pass) by 2 scales every product and sum by exactly 2
     in binary floating point, so outputs must scale bit-exactly: a linearity check that
