@@ -94,7 +94,7 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
     {   // rows narrower than a wave: several rows per wave (a requested 8 or 16 wins when it fits)
-        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes) : 0);
+        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes, false) : 0);
         if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 0}; return true; }
     }
     if (tpr_ok(tpr)) {
@@ -122,7 +122,7 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
     {   // rows narrower than a wave: several rows per wave, always 512-thread workgroups
-        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes) : 0);
+        const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes, true) : 0);
         if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 512}; return true; }
     }
     if (tpr_ok(tpr)) {

@@ -59,6 +59,7 @@ hipError_t narrow_by_items(int items, const BwdArgs& a, hipStream_t s) {
     switch (items) {
         case 1: return run_narrow<TPR, 1>(a, s);
         case 2: return run_narrow<TPR, 2>(a, s);
+        case 3: return run_narrow<TPR, 3>(a, s);
         case 4: return run_narrow<TPR, 4>(a, s);
         default: return hipErrorInvalidValue;
     }
@@ -96,6 +97,7 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
     if (cfg.vec != kVec) return hipErrorInvalidValue;
     if (cfg.tpr == 8 && cfg.block == 512) return narrow_by_items<8>(cfg.items, a, s);
     if (cfg.tpr == 16 && cfg.block == 512) return narrow_by_items<16>(cfg.items, a, s);
+    if (cfg.tpr == 32 && cfg.block == 512) return narrow_by_items<32>(cfg.items, a, s);
     if (cfg.block == 1024) return by_tpr<1024>(cfg.tpr, cfg.items, a, s);
     if (cfg.block == 512) return by_tpr<512>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;

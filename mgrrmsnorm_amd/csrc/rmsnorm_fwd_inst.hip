@@ -59,6 +59,7 @@ hipError_t narrow_by_items(int items, const FwdArgs& a, hipStream_t s) {
     switch (items) {
         case 1: return run_narrow<TPR, 1>(a, s);
         case 2: return run_narrow<TPR, 2>(a, s);
+        case 3: return run_narrow<TPR, 3>(a, s);
         case 4: return run_narrow<TPR, 4>(a, s);
         default: return hipErrorInvalidValue;
     }
@@ -69,6 +70,7 @@ hipError_t by_tpr(int tpr, int items, const FwdArgs& a, hipStream_t s) {
     switch (tpr) {
         case 8: return narrow_by_items<8>(items, a, s);
         case 16: return narrow_by_items<16>(items, a, s);
+        case 32: return narrow_by_items<32>(items, a, s);
         case 64: return by_items<VEC, 64>(items, a, s);
         case 128: return by_items<VEC, 128>(items, a, s);
         case 256: return by_items<VEC, 256>(items, a, s);

@@ -11,8 +11,8 @@
 // and dwords beyond it load 0 and store nothing).  A row of an odd number of 2-byte
 // elements ends in half a dword, which one lane moves with 2-byte accesses (RowTail).
 //
-// Narrow family: rows of at most 64 vectors whose pitch is a multiple of 16 bytes put 8 or
-// 16 lanes on a row, so that one wave carries 8 or 4 consecutive rows (see below).
+// Narrow family: rows of at most 128 vectors whose pitch is a multiple of 16 bytes put 8, 16
+// or 32 lanes on a row, so that one wave carries 8, 4 or 2 consecutive rows (see below).
 //
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
 // the row; used when the row does not fit the register-resident family (or on request).
@@ -88,11 +88,11 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
 }
 
 // =================================================================================
-// Narrow rows (at most 32 vectors, row pitch a multiple of 16 bytes): TPR = 8 or 16 lanes per
-// row, so a wave carries 64/TPR consecutive rows and a 256-thread workgroup 256/TPR.  One
-// buffer resource spans the wave's rows; lanes past the end of a row, and rows past the end
-// of the matrix, get an out-of-range offset (loads 0, stores nothing).  Row sums stay inside
-// the 16-lane DPP rows: no LDS, no barrier.
+// Narrow rows (row pitch a multiple of 16 bytes, at most 4 vectors per lane): TPR = 8, 16 or
+// 32 lanes per row, so a wave carries 64/TPR consecutive rows and a 256-thread workgroup
+// 256/TPR.  One buffer resource spans the wave's rows; lanes past the end of a row, and rows
+// past the end of the matrix, get an out-of-range offset (loads 0, stores nothing).  Row sums
+// stay inside the wave (DPP, plus v_readlane for 32 lanes): no LDS, no barrier.
 // =================================================================================
 constexpr u32 kOutOfRange = 0xFFFFFFF0u;
 

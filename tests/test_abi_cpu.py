@@ -140,7 +140,6 @@ def _launch_info(lib, backward, cols, dtype):
 @pytest.mark.parametrize("cols,dtype,fwd,bwd", [
     # 2-byte types: 8 elements per 16-byte vector
     (4096, 2, (0, 256, 2, 256), (0, 256, 2, 512)),      # metric shape: one row per 256-thread workgroup
-    (768, 2, (0, 64, 2, 256), (0, 64, 2, 512)),         # one wave per row
     (2048, 1, (0, 128, 2, 256), (0, 128, 2, 512)),
     (4100, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
     (5120, 1, (0, 512, 2, 512), (0, 256, 3, 512)),
@@ -148,12 +147,17 @@ def _launch_info(lib, backward, cols, dtype):
     (16384, 2, (0, 1024, 2, 1024), (0, 512, 4, 512)),
     (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
-    # rows narrower than a wave whose pitch is a multiple of 16 bytes: 8 or 16 lanes per row
+    # rows whose pitch is a multiple of 16 bytes share a wave: 8, 16 or 32 lanes per row;
+    # forward up to 4 vectors per lane (128 vectors), backward up to 2 (56 vectors)
     (64, 2, (0, 8, 1, 256), (0, 8, 1, 512)),            # 8 vectors: 8 rows per wave
-    (128, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # head-dimension 128
-    (256, 1, (0, 16, 2, 256), (0, 16, 2, 512)),
+    (128, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # head dimension 128
+    (256, 1, (0, 8, 4, 256), (0, 16, 2, 512)),
     (8, 2, (0, 8, 1, 256), (0, 8, 1, 512)),             # a single vector per row
-    (264, 2, (0, 64, 1, 256), (0, 64, 1, 512)),         # 33 vectors: one wave per row again
+    (264, 2, (0, 16, 3, 256), (0, 32, 2, 512)),         # 33 vectors
+    (512, 2, (0, 16, 4, 256), (0, 64, 1, 512)),         # 64 vectors: backward takes one wave per row
+    (768, 2, (0, 32, 3, 256), (0, 64, 2, 512)),
+    (1024, 1, (0, 32, 4, 256), (0, 64, 2, 512)),
+    (1032, 2, (0, 64, 3, 256), (0, 64, 3, 512)),        # 129 vectors: one wave per row
     (100, 2, (0, 64, 1, 256), (0, 64, 1, 512)),         # pitch 200 bytes: not a multiple of 16
     (64, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
     # fp32: 4 elements per vector, any width is 4-byte aligned

@@ -376,10 +376,10 @@ def test_backward_with_and_without_row_prefetch(prefetch, cols):
 
 
 @pytest.mark.parametrize("dtype", ALL)
-@pytest.mark.parametrize("tpr", [8, 16])
-@pytest.mark.parametrize("cols", [32, 64, 128, 256])
+@pytest.mark.parametrize("tpr", [8, 16, 32])
+@pytest.mark.parametrize("cols", [32, 72, 128, 192, 256, 512, 1000])
 def test_every_narrow_row_shape(dtype, tpr, cols):
-    """8 and 16 lanes per row with 1, 2 and 4 vectors per lane, whichever the automatic choice
+    """8, 16 and 32 lanes per row with 1 to 4 vectors per lane, whichever the automatic choice
     takes; a shape that does not fit the request falls back to the automatic one."""
     rows = 333
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=31 + cols)
