@@ -243,10 +243,13 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // 1/sqrt(v): the hardware estimate (about 1 ulp) refined by one Newton step, so that the
 // per-row scale, which the backward pass uses cubed, is good to about half an ulp.
+// v = +inf (a row holding an infinity, or squares that overflow fp32) gives 0 like rsqrtf:
+// the refinement would form inf * 0 there, so it is skipped.
 __device__ __forceinline__ float fast_rsqrt(float v) {
     const float y = __builtin_amdgcn_rsqf(v);
     const float e = __builtin_fmaf(-(v * y), y, 1.0f);  // 1 - v*y^2
-    return __builtin_fmaf(0.5f * y, e, y);
+    const float r = __builtin_fmaf(0.5f * y, e, y);
+    return v < __builtin_inff() ? r : y;
 }
 
 // sigmoid(g) = 1 / (1 + 2^(-g*log2(e))).  For g << 0 the power overflows to +inf and the

@@ -168,6 +168,34 @@ def test_zero_input_rows_give_zero_output_and_scaled_gradient():
     assert (dw == 0).all()
 
 
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("cols", [128, 4096])
+def test_non_finite_rows_behave_like_the_formula(dtype, cols):
+    """A NaN makes its own row NaN; an infinity (or squares that overflow fp32) drives the
+    row's scale to rsqrt(inf) = 0, so finite elements give 0 and the infinity itself NaN --
+    exactly what x * rsqrt(mean(x^2) + eps) * w gives (test_rmsnorm.py:55-56 in the
+    reference).  Rows that share a wave or a workgroup with such a row are untouched."""
+    rows = 64
+    x, _, w = U.rmsnorm_inputs(rows, cols, dtype, seed=77)
+    x[3, 5] = float("nan")
+    x[10, 7] = float("inf")
+    x[11, 0] = float("-inf")
+    if dtype != "fp16":
+        x[20, 9] = 3.0e38          # finite, but its square overflows fp32
+    xd, wd = _dev(x, w)
+    y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    xf, wf = xd.float(), wd.float()
+    want = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + EPS) * wf).to(U.DTYPES[dtype])
+    assert torch.equal(torch.isnan(y), torch.isnan(want))
+    assert torch.isnan(y[3]).all() and torch.isnan(y[10, 7]) and torch.isnan(y[11, 0])
+    assert (y[10, :7] == 0).all() and (y[10, 8:] == 0).all() and float(s[10]) == 0.0
+    if dtype != "fp16":
+        assert (y[20] == 0).all() and float(s[20]) == 0.0
+    clean = [r for r in range(rows) if r not in (3, 10, 11, 20)]
+    y_ref, *_ = U.rmsnorm_reference(x[clean], None, w, EPS, dtype)
+    U.assert_matches(y[clean], y_ref, dtype, "rows next to non-finite ones")
+
+
 # --------------------------------------------------------------------------- determinism
 
 @pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 2000, 5120), ("fp32", 777, 1000),
