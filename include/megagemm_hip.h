@@ -140,8 +140,8 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
  * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
  * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
  * workgroup per row, *vectors_per_thread = 0).  *threads_per_row below 64 means that
- * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB whose pitch
- * is a multiple of 16 bytes).
+ * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
+ * 640 bytes when the pitch is not a multiple of 16 bytes).
  */
 int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
                            int* vectors_per_thread, int* workgroup_threads);
@@ -157,8 +157,7 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
 /*
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
- * rows of at most 4 vectors per thread whose pitch is a multiple of 16 bytes; -1 = never
- * fewer than 64), "fwd_items" (target
+ * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
  * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
  * the current one; -1 = automatic), "swiglu_unroll",

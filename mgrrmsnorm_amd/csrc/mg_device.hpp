@@ -126,6 +126,47 @@ __device__ __forceinline__ void store_item(rsrc_t r, int lir, int i, const Words
 }
 
 // ---------------------------------------------------------------------------------
+// Rows packed back to back under one buffer resource (several rows per wave): a 16-byte
+// vector that starts `pos` bytes into a row of `row_bytes` may run past the end of its row
+// into the next one.  `rem` = row_bytes - pos is what the row still holds from there (as an
+// unsigned difference it wraps to a huge value for a lane that has no vector in the row,
+// which reads as "nothing to trim": such a lane's offset is out of range anyway).
+// trim_row_vector() zeroes the words beyond the row after a plain 16-byte load -- it only
+// touches registers, so it can run long after the load was issued -- and puts in `tail_bits`
+// where a row of an odd number of 2-byte elements ends in half a dword (the lane holding that
+// word fetches the element with a 2-byte load of its own).  store_row_vector() stores only
+// what belongs to the row.
+// ---------------------------------------------------------------------------------
+__device__ __forceinline__ void trim_row_vector(Words<4>& v, u32 rem, u32 tail_bits) {
+    const int r = rem < 16u ? (int)rem : 16;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int left = r - 4 * j;
+        v.v[j] = left >= 4 ? v.v[j] : (left == 2 ? tail_bits : 0u);
+    }
+}
+
+template <int POLICY>
+__device__ __forceinline__ void store_row_vector(rsrc_t r, u32 off, u32 rem, const Words<4>& w) {
+    if (rem >= 16u) {
+        buf_store<4, POLICY>(r, off, w);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int left = (int)rem - 4 * j;
+            if (left >= 4) __builtin_amdgcn_raw_buffer_store_b32(w.v[j], r, (int)(off + 4u * j), 0, POLICY);
+            else if (left == 2)
+                __builtin_amdgcn_raw_buffer_store_b16((unsigned short)(w.v[j] & 0xffffu), r, (int)(off + 4u * j), 0, POLICY);
+        }
+    }
+}
+
+template <int POLICY>
+__device__ __forceinline__ u32 load_b16(rsrc_t r, u32 off) {
+    return (u32)__builtin_amdgcn_raw_buffer_load_b16(r, (int)off, 0, POLICY);
+}
+
+// ---------------------------------------------------------------------------------
 // Element traits: PER_WORD elements per 32-bit word, conversion to/from fp32.
 // fp32 -> fp16/bf16 uses the hardware round-to-nearest-even converts
 // (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32); never the round-toward-zero pack.

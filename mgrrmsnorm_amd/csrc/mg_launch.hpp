@@ -33,21 +33,23 @@ constexpr bool bwd_cfg_ok(int esize, int tpr, int items, int block) {
 }
 constexpr bool tpr_ok(int tpr) { return tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024; }
 
-// Rows whose pitch is a multiple of 16 bytes can share a wave: 8, 16 or 32 lanes per row and
-// up to 4 vectors per lane (rows of at most 128 vectors = 2 KiB).
+// Rows of at most 128 vectors can share a wave: 8, 16 or 32 lanes per row and up to 4
+// vectors per lane.
 constexpr bool narrow_tpr(int tpr) { return tpr == 8 || tpr == 16 || tpr == 32; }
 constexpr int narrow_items(long row_bytes, int tpr) {   // 0 = does not fit
-    if (!narrow_tpr(tpr) || row_bytes % kVec != 0) return 0;
-    const long need = (row_bytes / kVec + tpr - 1) / tpr;
+    if (!narrow_tpr(tpr)) return 0;
+    const long need = ((row_bytes + kVec - 1) / kVec + tpr - 1) / tpr;
     return need <= 4 ? (int)need : 0;
 }
 // Default use, from sweeps over row widths on MI355X (0 = one or more waves per row).
-// Forward: the fewest lanes that hold the row in 4 vectors each, up to 128 vectors.
-// Backward (which also carries dy, a prefetched row and the dW sums): 2 vectors each, up to
-// 56 vectors; from there on one wave per row is as fast.
+// Pitch a multiple of 16 bytes -- forward: the fewest lanes that hold the row in 4 vectors
+// each, up to 128 vectors; backward (which also carries dy, a prefetched row and the dW
+// sums): 2 vectors each, up to 56 vectors; from there on one wave per row is as fast.
+// Other pitches (a row's last vector is moved in pieces and rows share cache lines) gain
+// only while a row is short: up to 40 vectors, with the split that measured best.
 constexpr int narrow_default_tpr(long row_bytes, bool backward) {
-    if (row_bytes % kVec != 0) return 0;
-    const long nvec = row_bytes / kVec;
+    const long nvec = (row_bytes + kVec - 1) / kVec;
+    if (row_bytes % kVec != 0) return nvec <= 24 ? 8 : (nvec <= 32 ? 32 : (nvec <= 40 ? 16 : 0));
     if (backward) return nvec <= 16 ? 8 : (nvec <= 32 ? 16 : (nvec <= 56 ? 32 : 0));
     return nvec <= 32 ? 8 : (nvec <= 64 ? 16 : (nvec <= 128 ? 32 : 0));
 }

@@ -45,9 +45,9 @@ hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
     }
 }
 
-template <int TPR, int ITEMS>
+template <int TPR, int ITEMS, bool RAGGED>
 hipError_t run_narrow(const BwdArgs& a, hipStream_t s) {
-    rmsnorm_bwd_narrow<elem_t, TPR, ITEMS><<<dim3((unsigned)a.num_partials), dim3(512), 0, s>>>(
+    rmsnorm_bwd_narrow<elem_t, TPR, ITEMS, RAGGED><<<dim3((unsigned)a.num_partials), dim3(512), 0, s>>>(
         (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
         a.rows, a.cols, 1.0f / (float)a.cols);
     return hipGetLastError();
@@ -56,11 +56,12 @@ hipError_t run_narrow(const BwdArgs& a, hipStream_t s) {
 template <int TPR>
 hipError_t narrow_by_items(int items, const BwdArgs& a, hipStream_t s) {
     if (narrow_items((long)a.cols * (long)sizeof(elem_t), TPR) != items) return hipErrorInvalidValue;
+    const bool ragged = ((long)a.cols * (long)sizeof(elem_t)) % kVec != 0;
     switch (items) {
-        case 1: return run_narrow<TPR, 1>(a, s);
-        case 2: return run_narrow<TPR, 2>(a, s);
-        case 3: return run_narrow<TPR, 3>(a, s);
-        case 4: return run_narrow<TPR, 4>(a, s);
+        case 1: return ragged ? run_narrow<TPR, 1, true>(a, s) : run_narrow<TPR, 1, false>(a, s);
+        case 2: return ragged ? run_narrow<TPR, 2, true>(a, s) : run_narrow<TPR, 2, false>(a, s);
+        case 3: return ragged ? run_narrow<TPR, 3, true>(a, s) : run_narrow<TPR, 3, false>(a, s);
+        case 4: return ragged ? run_narrow<TPR, 4, true>(a, s) : run_narrow<TPR, 4, false>(a, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -11,8 +11,8 @@
 // and dwords beyond it load 0 and store nothing).  A row of an odd number of 2-byte
 // elements ends in half a dword, which one lane moves with 2-byte accesses (RowTail).
 //
-// Narrow family: rows of at most 128 vectors whose pitch is a multiple of 16 bytes put 8, 16
-// or 32 lanes on a row, so that one wave carries 8, 4 or 2 consecutive rows (see below).
+// Narrow family: rows of at most 128 vectors put 8, 16 or 32 lanes on a row, so that one
+// wave carries 8, 4 or 2 consecutive rows (see below).
 //
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
 // the row; used when the row does not fit the register-resident family (or on request).
@@ -88,21 +88,58 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
 }
 
 // =================================================================================
-// Narrow rows (row pitch a multiple of 16 bytes, at most 4 vectors per lane): TPR = 8, 16 or
-// 32 lanes per row, so a wave carries 64/TPR consecutive rows and a 256-thread workgroup
-// 256/TPR.  One buffer resource spans the wave's rows; lanes past the end of a row, and rows
-// past the end of the matrix, get an out-of-range offset (loads 0, stores nothing).  Row sums
-// stay inside the wave (DPP, plus v_readlane for 32 lanes): no LDS, no barrier.
+// Narrow rows (at most 4 vectors per lane): TPR = 8, 16 or 32 lanes per row, so a wave
+// carries 64/TPR consecutive rows and a 256-thread workgroup 256/TPR.  One buffer resource
+// spans the wave's rows; lanes past the end of a row, and rows past the end of the matrix,
+// get an out-of-range offset (loads 0, stores nothing).  Row sums stay inside the wave (DPP,
+// plus v_readlane for 32 lanes): no LDS, no barrier.  RAGGED = the row pitch is not a
+// multiple of 16 bytes: the last vector of a row then reaches into the next row and is
+// trimmed to its own row on load and on store (load_row_vector / store_row_vector).
 // =================================================================================
 constexpr u32 kOutOfRange = 0xFFFFFFF0u;
 
-template <typename T, int TPR, int ITEMS>
+// Activations of ragged rows take the default cache policy: a row's last vector is stored in
+// pieces, and lines shared by two rows are written by two instructions; the L2 merges those
+// writes, whereas non-temporal ones reach memory piecemeal (measured: 2.2 against 4.7 TB/s
+// at 100 bf16 columns).
+template <bool RAGGED> constexpr int kNarrowPolicy = RAGGED ? kKeep : kStream;
+
+// Where this lane's vectors sit in a narrow row, fixed for the whole kernel.
+template <int TPR, int ITEMS>
+struct NarrowLane {
+    u32 off[ITEMS];   // byte offset under the wave's buffer resource, or out of range
+    u32 woff[ITEMS];  // byte offset in the weight row, or out of range
+    u32 rem[ITEMS];   // bytes the row still holds from the vector's start (ragged rows)
+    u32 tail_off;     // where the row's last 2-byte element is, for the lane that patches it in
+    bool owns_tail;   // the row ends in half a dword and this lane holds that word
+};
+
+template <typename T, int TPR, int ITEMS, bool RAGGED>
+__device__ __forceinline__ NarrowLane<TPR, ITEMS> narrow_lane(int sub, int lir, u32 row_bytes) {
+    NarrowLane<TPR, ITEMS> p;
+    const u32 nvec = (row_bytes + 15u) / 16u;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const u32 vec = (u32)(lir + i * TPR);
+        p.off[i] = vec < nvec ? (u32)sub * row_bytes + vec * 16u : kOutOfRange;
+        p.woff[i] = vec < nvec ? vec * 16u : kOutOfRange;
+        p.rem[i] = row_bytes - vec * 16u;
+    }
+    p.owns_tail = false;
+    p.tail_off = row_bytes - 2u;
+    if constexpr (RAGGED && sizeof(T) == 2)
+        p.owns_tail = (row_bytes & 2u) != 0 && (u32)lir == ((row_bytes - 1u) / 16u) % TPR;
+    return p;
+}
+
+template <typename T, int TPR, int ITEMS, bool RAGGED>
 __global__ void __launch_bounds__(256)
 rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
                    const T* __restrict__ w, long rows, int cols, float eps, float inv_cols, int xcd_group) {
     constexpr int RPW = kWave / TPR;   // rows per wave
     constexpr int RPB = 256 / TPR;     // rows per workgroup
     constexpr int EPV = 16 / (int)sizeof(T);
+    constexpr int POL = kNarrowPolicy<RAGGED>;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int lane = tid & (kWave - 1);
@@ -112,20 +149,28 @@ rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __re
     const long left = rows - row0;
     const u32 live_rows = left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
     const u32 row_bytes = (u32)cols * (u32)sizeof(T);
-    const u32 nvec = row_bytes / 16u;
     const long base = live_rows ? row0 * (long)cols : 0;
     const rsrc_t rx = make_rsrc(x + base, live_rows * row_bytes);
     const rsrc_t ry = make_rsrc(y + base, live_rows * row_bytes);
     const rsrc_t rw = make_rsrc(w, row_bytes);
+    const NarrowLane<TPR, ITEMS> p = narrow_lane<T, TPR, ITEMS, RAGGED>(sub, lir, row_bytes);
 
     Words<4> xv[ITEMS], wv[ITEMS];
-    u32 off[ITEMS];
+    u32 x_tail = 0, w_tail = 0;
 #pragma unroll
-    for (int i = 0; i < ITEMS; ++i) {
-        const u32 vec = (u32)(lir + i * TPR);
-        off[i] = vec < nvec ? (u32)sub * row_bytes + vec * 16u : kOutOfRange;
-        xv[i] = buf_load<4, kStream>(rx, off[i]);
-        wv[i] = buf_load<4, kKeep>(rw, vec < nvec ? vec * 16u : kOutOfRange);
+    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<4, POL>(rx, p.off[i]);
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<4, kKeep>(rw, p.woff[i]);
+    if constexpr (RAGGED) {
+        if (p.owns_tail) {
+            x_tail = load_b16<POL>(rx, (u32)sub * row_bytes + p.tail_off);
+            w_tail = load_b16<kKeep>(rw, p.tail_off);
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            trim_row_vector(xv[i], p.rem[i], x_tail);
+            trim_row_vector(wv[i], p.rem[i], w_tail);
+        }
     }
     float ss = 0.0f;
 #pragma unroll
@@ -145,16 +190,18 @@ rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __re
         unpack_vec<T, 4>(wv[i], wf);
 #pragma unroll
         for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
-        buf_store<4, kStream>(ry, off[i], pack_vec<T, 4>(o));
+        if constexpr (RAGGED) store_row_vector<POL>(ry, p.off[i], p.rem[i], pack_vec<T, 4>(o));
+        else buf_store<4, POL>(ry, p.off[i], pack_vec<T, 4>(o));
     }
 }
 
 // Backward pass 1 for narrow rows: persistent grid of 512-thread workgroups; each wave walks
 // groups of 64/TPR consecutive rows (group g of wave q: rows (g*Q + q)*RPW ..., Q = all waves),
-// prefetching the next group.  dW: per lane in registers, then across the rows of a wave by
-// lane shuffles, then across the 8 waves in wave order through LDS; one partial row per
-// workgroup.
-template <typename T, int TPR, int ITEMS>
+// prefetching the next group (ragged rows are trimmed when the data is used, not when it is
+// requested, so the prefetch stays in flight).  dW: per lane in registers, then across the
+// rows of a wave by lane shuffles, then across the 8 waves in wave order through LDS; one
+// partial row per workgroup.
+template <typename T, int TPR, int ITEMS, bool RAGGED>
 __global__ void __launch_bounds__(512)
 rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                    const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
@@ -164,6 +211,7 @@ rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, cons
     constexpr int RPW = kWave / TPR;
     constexpr int EPV = 16 / (int)sizeof(T);
     constexpr int COVER = TPR * ITEMS * EPV;   // columns one row's lanes cover (>= cols)
+    constexpr int POL = kNarrowPolicy<RAGGED>;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int lane = tid & (kWave - 1);
@@ -174,7 +222,8 @@ rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, cons
     const long ngroups = (rows + RPW - 1) / RPW;            // groups of RPW rows in the matrix
     const long n_it = (ngroups + nwaves - 1) / nwaves;
     const u32 row_bytes = (u32)cols * (u32)sizeof(T);
-    const u32 nvec = row_bytes / 16u;
+    const NarrowLane<TPR, ITEMS> p = narrow_lane<T, TPR, ITEMS, RAGGED>(sub, lir, row_bytes);
+    const u32 tail_at = (u32)sub * row_bytes + p.tail_off;
 
     float acc[ITEMS][EPV];
 #pragma unroll
@@ -183,14 +232,15 @@ rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, cons
         for (int k = 0; k < EPV; ++k) acc[i][k] = 0.0f;
 
     Words<4> wv[ITEMS];
-    u32 voff[ITEMS];   // offset inside the wave's rows, or out of range
     {
         const rsrc_t rw = make_rsrc(w, row_bytes);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) {
-            const u32 vec = (u32)(lir + i * TPR);
-            voff[i] = vec < nvec ? (u32)sub * row_bytes + vec * 16u : kOutOfRange;
-            wv[i] = buf_load<4, kKeep>(rw, vec < nvec ? vec * 16u : kOutOfRange);
+        for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<4, kKeep>(rw, p.woff[i]);
+        if constexpr (RAGGED) {
+            u32 w_tail = 0;
+            if (p.owns_tail) w_tail = load_b16<kKeep>(rw, p.tail_off);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) trim_row_vector(wv[i], p.rem[i], w_tail);
         }
     }
 
@@ -198,38 +248,45 @@ rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, cons
         const long left = rows - row0;
         return left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
     };
-
-    Words<4> xv[ITEMS], gv[ITEMS];
-    long row0 = q * RPW;
-    u32 live = live_rows_of(row0);
-    float s = 0.0f;
-    {
+    // requests the x and dy vectors (and the odd last elements) of the rows from row0 on
+    auto request = [&](long row0, u32 live, Words<4> (&xo)[ITEMS], Words<4> (&go)[ITEMS], u32& xt, u32& gt, float& so) {
         const long base = live ? row0 * (long)cols : 0;
         const rsrc_t rx = make_rsrc(x + base, live * row_bytes);
         const rsrc_t rg = make_rsrc(dy + base, live * row_bytes);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<4, kStream>(rx, voff[i]);
+        for (int i = 0; i < ITEMS; ++i) xo[i] = buf_load<4, POL>(rx, p.off[i]);
 #pragma unroll
-        for (int i = 0; i < ITEMS; ++i) gv[i] = buf_load<4, kStream>(rg, voff[i]);
-        if ((u32)sub < live) s = inv_rms[row0 + sub];
-    }
+        for (int i = 0; i < ITEMS; ++i) go[i] = buf_load<4, POL>(rg, p.off[i]);
+        xt = 0; gt = 0;
+        if constexpr (RAGGED) {
+            if (p.owns_tail) { xt = load_b16<POL>(rx, tail_at); gt = load_b16<POL>(rg, tail_at); }
+        }
+        so = 0.0f;
+        if ((u32)sub < live) so = inv_rms[row0 + sub];
+    };
+
+    Words<4> xv[ITEMS], gv[ITEMS];
+    u32 x_tail, g_tail;
+    long row0 = q * RPW;
+    u32 live = live_rows_of(row0);
+    float s;
+    request(row0, live, xv, gv, x_tail, g_tail, s);
 
     for (long it = 0; it < n_it; ++it) {
         const long nrow0 = row0 + nwaves * RPW;
         const u32 nlive = live_rows_of(nrow0);
         Words<4> nxv[ITEMS], ngv[ITEMS];
-        float ns = 0.0f;
-        {
-            const long nbase = nlive ? nrow0 * (long)cols : 0;
-            const rsrc_t rx = make_rsrc(x + nbase, nlive * row_bytes);
-            const rsrc_t rg = make_rsrc(dy + nbase, nlive * row_bytes);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) nxv[i] = buf_load<4, kStream>(rx, voff[i]);
-#pragma unroll
-            for (int i = 0; i < ITEMS; ++i) ngv[i] = buf_load<4, kStream>(rg, voff[i]);
-            if ((u32)sub < nlive) ns = inv_rms[nrow0 + sub];
-        }
+        u32 nx_tail, ng_tail;
+        float ns;
+        request(nrow0, nlive, nxv, ngv, nx_tail, ng_tail, ns);
 
+        if constexpr (RAGGED) {
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) {
+                trim_row_vector(xv[i], p.rem[i], x_tail);
+                trim_row_vector(gv[i], p.rem[i], g_tail);
+            }
+        }
         float a = 0.0f;
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
@@ -257,11 +314,13 @@ rmsnorm_bwd_narrow(T* __restrict__ dx, float* __restrict__ dw_part, int ld, cons
                 unpack_vec<T, 4>(wv[i], wf);
 #pragma unroll
                 for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
-                buf_store<4, kStream>(rd, voff[i], pack_vec<T, 4>(o));
+                if constexpr (RAGGED) store_row_vector<POL>(rd, p.off[i], p.rem[i], pack_vec<T, 4>(o));
+                else buf_store<4, POL>(rd, p.off[i], pack_vec<T, 4>(o));
             }
         }
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+        x_tail = nx_tail; g_tail = ng_tail;
         row0 = nrow0; live = nlive; s = ns;
     }
 

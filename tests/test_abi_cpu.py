@@ -147,7 +147,7 @@ def _launch_info(lib, backward, cols, dtype):
     (16384, 2, (0, 1024, 2, 1024), (0, 512, 4, 512)),
     (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
-    # rows whose pitch is a multiple of 16 bytes share a wave: 8, 16 or 32 lanes per row;
+    # rows of up to 2 KiB share a wave: 8, 16 or 32 lanes per row;
     # forward up to 4 vectors per lane (128 vectors), backward up to 2 (56 vectors)
     (64, 2, (0, 8, 1, 256), (0, 8, 1, 512)),            # 8 vectors: 8 rows per wave
     (128, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # head dimension 128
@@ -158,11 +158,13 @@ def _launch_info(lib, backward, cols, dtype):
     (768, 2, (0, 32, 3, 256), (0, 64, 2, 512)),
     (1024, 1, (0, 32, 4, 256), (0, 64, 2, 512)),
     (1032, 2, (0, 64, 3, 256), (0, 64, 3, 512)),        # 129 vectors: one wave per row
-    (100, 2, (0, 64, 1, 256), (0, 64, 1, 512)),         # pitch 200 bytes: not a multiple of 16
+    (100, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # pitch 200 bytes: the last vector of a row is trimmed
+    (299, 1, (0, 16, 3, 256), (0, 16, 3, 512)),         # 598 bytes, rows only 2-byte aligned
+    (999, 1, (0, 64, 2, 256), (0, 64, 2, 512)),         # 1998 bytes: too long for that to pay
     (64, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
     # fp32: 4 elements per vector, any width is 4-byte aligned
     (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
-    (33, 0, (0, 64, 1, 256), (0, 64, 1, 512)),
+    (33, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
     (16384, 0, (0, 1024, 4, 1024), (0, 512, 8, 512)),
 ])
 def test_launch_shapes(lib, cols, dtype, fwd, bwd):

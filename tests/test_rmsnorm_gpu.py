@@ -69,6 +69,9 @@ SHAPES = [
     (5000, 200),     # 25 vectors over 16 lanes
     (3, 32),
     (70000, 16),     # more rows than the backward grid has row slots at once
+    (4001, 100),     # pitch 200 bytes: a row's last vector reaches into the next row and is trimmed
+    (3001, 127),     # odd width: rows 2-byte aligned, each ends in half a dword
+    (999, 299),
 ]
 
 
@@ -405,7 +408,7 @@ def test_backward_with_and_without_row_prefetch(prefetch, cols):
 
 @pytest.mark.parametrize("dtype", ALL)
 @pytest.mark.parametrize("tpr", [8, 16, 32])
-@pytest.mark.parametrize("cols", [32, 72, 128, 192, 256, 512, 1000])
+@pytest.mark.parametrize("cols", [32, 72, 128, 192, 256, 512, 1000, 100, 127, 299, 45])   # the last four: ragged pitches
 def test_every_narrow_row_shape(dtype, tpr, cols):
     """8, 16 and 32 lanes per row with 1 to 4 vectors per lane, whichever the automatic choice
     takes; a shape that does not fit the request falls back to the automatic one."""
