@@ -237,6 +237,7 @@ SWEEP = [
     # rows narrower than a wave (per-head QK-norm widths): several rows per wave
     "rmsnorm_fwd_bwd_2097152x64_bf16", "rmsnorm_fwd_bwd_1048576x128_bf16", "rmsnorm_fwd_bwd_524288x256_bf16",
     "rmsnorm_fwd_bwd_1048576x64_fp32",
+    "rmsnorm_fwd_bwd_1342144x100_bf16",   # pitch 200 bytes: not a multiple of 16
     "swiglu_fwd_bwd_8192x11008_bf16",
 ]
 
