@@ -117,7 +117,9 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
 // Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  Measured on MI355X,
 // about 64 KiB of loads in flight per compute unit saturates HBM and more waves than that
 // only add contention, so: the most threads per row (fewest vectors per thread) that still
-// keep (row slots) x (row bytes) x (x and dy) x (current + prefetched row) >= 48 KiB.
+// keep (row slots) x (row bytes) x (x and dy) x (current + prefetched row) >= 36 KiB
+// (sweep over 576...10240 columns: two vectors per thread beat three at half the threads by
+// 4-10 %, e.g. 1280 columns 6.3 against 5.7 TB/s, while 4096 columns still want 256 x 2).
 bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
@@ -140,7 +142,7 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         for (int t = b; t >= 64; t /= 2) {
             const int need = round_items(ceil_div(nvec, t));
             const long in_flight = (long)(b / t) * row_bytes * 4;
-            if (in_flight >= 48 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+            if (in_flight >= 36 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
         }
         for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
             const int need = round_items(ceil_div(nvec, t));

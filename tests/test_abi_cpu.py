@@ -142,7 +142,7 @@ def _launch_info(lib, backward, cols, dtype):
     (4096, 2, (0, 256, 2, 256), (0, 256, 2, 512)),      # metric shape: one row per 256-thread workgroup
     (2048, 1, (0, 128, 2, 256), (0, 128, 2, 512)),
     (4100, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
-    (5120, 1, (0, 512, 2, 512), (0, 256, 3, 512)),
+    (5120, 1, (0, 512, 2, 512), (0, 512, 2, 512)),
     (8192, 2, (0, 512, 2, 512), (0, 512, 2, 512)),
     (16384, 2, (0, 1024, 2, 1024), (0, 1024, 2, 1024)),
     (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
