@@ -376,6 +376,15 @@ static int check_swiglu(const char* fn, int64_t M, int64_t H, int dtype) {
     return MG_OK;
 }
 
+// Aligned 16-byte vectors when the half-row pitch and every base allow it; otherwise 16-byte
+// vectors at any alignment (a row of [gate | up] must stay below 2^31 bytes for their 32-bit
+// offsets); one element per thread on request or for such enormous rows.
+static int swiglu_mode(int64_t half_row_bytes, bool bases_aligned) {
+    if (opt_force_generic.load() != 0) return kSwigluElementwise;
+    if (half_row_bytes % 16 == 0 && bases_aligned) return kSwigluAligned;
+    return 2 * half_row_bytes < (1LL << 31) ? kSwigluRagged : kSwigluElementwise;
+}
+
 static int swiglu_unroll(int dflt, int maxv) {
     int u = opt_swiglu_unroll.load();
     if (u == 1 || u == 2 || u == 4 || (u == 8 && maxv >= 8)) return u;
@@ -390,8 +399,8 @@ int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void
     const int es = esize_of(dtype);
     if (!aligned(h, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: a pointer is not aligned to its element size");
-    const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(h, 16) && aligned(gu, 16);
-    hipError_t e = launch_swiglu_fwd(dtype, vec, swiglu_unroll(1, 8), xcd_group_or(kXcdGroupStreaming), h, gu, (long)M, (long)H, (hipStream_t)stream);
+    const int mode = swiglu_mode(H * es, aligned(h, 16) && aligned(gu, 16));
+    hipError_t e = launch_swiglu_fwd(dtype, mode, swiglu_unroll(1, 8), xcd_group_or(kXcdGroupStreaming), h, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_fwd: launch", e);
     return MG_OK;
 }
@@ -405,10 +414,9 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
     const int es = esize_of(dtype);
     if (!aligned(dgu, es) || !aligned(dh, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_bwd: a pointer is not aligned to its element size");
-    const bool vec = opt_force_generic.load() == 0 && (H * es) % 16 == 0 && aligned(dgu, 16) && aligned(dh, 16) &&
-                     aligned(gu, 16);
+    const int mode = swiglu_mode(H * es, aligned(dgu, 16) && aligned(dh, 16) && aligned(gu, 16));
     hipError_t e =
-        launch_swiglu_bwd(dtype, vec, swiglu_unroll(1, 4), xcd_group_or(kXcdGroupStreaming), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
+        launch_swiglu_bwd(dtype, mode, swiglu_unroll(1, 4), xcd_group_or(kXcdGroupStreaming), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_bwd: launch", e);
     return MG_OK;
 }

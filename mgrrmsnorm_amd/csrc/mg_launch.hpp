@@ -76,13 +76,15 @@ hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const 
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s);
 hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s);
 
-// SwiGLU: `vec` = true takes the 16-byte kernels (requires H*sizeof(T) % 16 == 0 and
-// 16-byte aligned bases).  rows*H per launch must stay below 2^31 units (vectors or elements).
-// Upper bound on units per launch (default and maximum 2^31); larger inputs are split by rows.
+// SwiGLU kernel families: aligned 16-byte vectors (needs H*sizeof(T) % 16 == 0 and 16-byte
+// aligned bases), 16-byte vectors at any alignment with ragged half rows, or one element per
+// thread.  rows*H per launch stays below 2^31 units (vectors or elements); larger inputs are
+// split by rows, as are inputs above the "swiglu_max_units" option.
+constexpr int kSwigluElementwise = 0, kSwigluAligned = 1, kSwigluRagged = 2;
 void set_swiglu_max_units(long units);
-hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, int xcd_group, void* h, const void* gu, long M, long H,
+hipError_t launch_swiglu_fwd(int dtype, int mode, int unroll, int xcd_group, void* h, const void* gu, long M, long H,
                              hipStream_t s);
-hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, int xcd_group, void* dgu, const void* dh, const void* gu,
+hipError_t launch_swiglu_bwd(int dtype, int mode, int unroll, int xcd_group, void* dgu, const void* dh, const void* gu,
                              long M, long H, hipStream_t s);
 
 }  // namespace mg

@@ -67,6 +67,49 @@ hipError_t bwd_vec(int xg, void* dgu, const void* dh, const void* gu, long M, lo
     return hipSuccess;
 }
 
+// rows one launch of the ragged kernels may cover: as above, and all byte offsets below 2^31
+long ragged_rows_per_launch(long nvr, long half_bytes) {
+    long r = rows_per_launch_for(nvr);
+    const long by_bytes = (1L << 31) / (2 * half_bytes);
+    if (r > by_bytes) r = by_bytes;
+    return r < 1 ? 1 : r;
+}
+
+template <typename T>
+hipError_t fwd_ragged(int xg, void* h, const void* gu, long M, long H, hipStream_t s) {
+    const long half_bytes = H * (long)sizeof(T);
+    const long nvr = (half_bytes + 15) / 16;
+    const long rows_per_launch = ragged_rows_per_launch(nvr, half_bytes);
+    const FastDiv fd = make_fastdiv((uint32_t)nvr);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * nvr);
+        swiglu_fwd_ragged<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+            (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, (uint32_t)m, total, (uint32_t)half_bytes, fd, xg);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t bwd_ragged(int xg, void* dgu, const void* dh, const void* gu, long M, long H, hipStream_t s) {
+    const long half_bytes = H * (long)sizeof(T);
+    const long nvr = (half_bytes + 15) / 16;
+    const long rows_per_launch = ragged_rows_per_launch(nvr, half_bytes);
+    const FastDiv fd = make_fastdiv((uint32_t)nvr);
+    for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
+        const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
+        const uint32_t total = (uint32_t)(m * nvr);
+        swiglu_bwd_ragged<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+            (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, (uint32_t)m, total,
+            (uint32_t)half_bytes, fd, xg);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 template <typename T>
 hipError_t fwd_gen(void* h, const void* gu, long M, long H, hipStream_t s) {
     const long rows_per_launch = rows_per_launch_for(H);
@@ -98,8 +141,9 @@ hipError_t bwd_gen(void* dgu, const void* dh, const void* gu, long M, long H, hi
 }
 
 template <typename T>
-hipError_t fwd_t(bool vec, int unroll, int xg, void* h, const void* gu, long M, long H, hipStream_t s) {
-    if (!vec) return fwd_gen<T>(h, gu, M, H, s);
+hipError_t fwd_t(int mode, int unroll, int xg, void* h, const void* gu, long M, long H, hipStream_t s) {
+    if (mode == kSwigluElementwise) return fwd_gen<T>(h, gu, M, H, s);
+    if (mode == kSwigluRagged) return fwd_ragged<T>(xg, h, gu, M, H, s);
     switch (unroll) {
         case 1: return fwd_vec<T, 1>(xg, h, gu, M, H, s);
         case 2: return fwd_vec<T, 2>(xg, h, gu, M, H, s);
@@ -110,9 +154,10 @@ hipError_t fwd_t(bool vec, int unroll, int xg, void* h, const void* gu, long M, 
 }
 
 template <typename T>
-hipError_t bwd_t(bool vec, int unroll, int xg, void* dgu, const void* dh, const void* gu, long M, long H,
+hipError_t bwd_t(int mode, int unroll, int xg, void* dgu, const void* dh, const void* gu, long M, long H,
                  hipStream_t s) {
-    if (!vec) return bwd_gen<T>(dgu, dh, gu, M, H, s);
+    if (mode == kSwigluElementwise) return bwd_gen<T>(dgu, dh, gu, M, H, s);
+    if (mode == kSwigluRagged) return bwd_ragged<T>(xg, dgu, dh, gu, M, H, s);
     switch (unroll) {
         case 1: return bwd_vec<T, 1>(xg, dgu, dh, gu, M, H, s);
         case 2: return bwd_vec<T, 2>(xg, dgu, dh, gu, M, H, s);
@@ -127,22 +172,22 @@ void set_swiglu_max_units(long units) {
     g_max_units.store(units >= 1 && units <= kMaxUnitsPerLaunchDefault ? units : kMaxUnitsPerLaunchDefault);
 }
 
-hipError_t launch_swiglu_fwd(int dtype, bool vec, int unroll, int xg, void* h, const void* gu, long M, long H,
+hipError_t launch_swiglu_fwd(int dtype, int mode, int unroll, int xg, void* h, const void* gu, long M, long H,
                              hipStream_t s) {
     switch (dtype) {
-        case MG_F32: return fwd_t<float>(vec, unroll, xg, h, gu, M, H, s);
-        case MG_F16: return fwd_t<half_t>(vec, unroll, xg, h, gu, M, H, s);
-        case MG_BF16: return fwd_t<bf16_t>(vec, unroll, xg, h, gu, M, H, s);
+        case MG_F32: return fwd_t<float>(mode, unroll, xg, h, gu, M, H, s);
+        case MG_F16: return fwd_t<half_t>(mode, unroll, xg, h, gu, M, H, s);
+        case MG_BF16: return fwd_t<bf16_t>(mode, unroll, xg, h, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }
 
-hipError_t launch_swiglu_bwd(int dtype, bool vec, int unroll, int xg, void* dgu, const void* dh, const void* gu,
+hipError_t launch_swiglu_bwd(int dtype, int mode, int unroll, int xg, void* dgu, const void* dh, const void* gu,
                              long M, long H, hipStream_t s) {
     switch (dtype) {
-        case MG_F32: return bwd_t<float>(vec, unroll, xg, dgu, dh, gu, M, H, s);
-        case MG_F16: return bwd_t<half_t>(vec, unroll, xg, dgu, dh, gu, M, H, s);
-        case MG_BF16: return bwd_t<bf16_t>(vec, unroll, xg, dgu, dh, gu, M, H, s);
+        case MG_F32: return bwd_t<float>(mode, unroll, xg, dgu, dh, gu, M, H, s);
+        case MG_F16: return bwd_t<half_t>(mode, unroll, xg, dgu, dh, gu, M, H, s);
+        case MG_BF16: return bwd_t<bf16_t>(mode, unroll, xg, dgu, dh, gu, M, H, s);
         default: return hipErrorInvalidValue;
     }
 }

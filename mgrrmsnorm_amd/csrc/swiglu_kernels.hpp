@@ -100,7 +100,82 @@ swiglu_bwd_vec(T* __restrict__ dgu, const T* __restrict__ dh, const T* __restric
     }
 }
 
-// Element-wise variants for H * sizeof(T) not a multiple of 16 or misaligned bases.
+// Any H and any element-aligned base: 16-byte buffer accesses at whatever alignment the row
+// gives them.  A half row of H elements is cut into nvr = ceil(H * sizeof(T) / 16) vectors;
+// the last one reaches past the half row (into the `up` half, the next row, or -- at the end
+// of the launch's rows -- out of the buffer, where loads return 0), which is harmless for
+// loads since nothing is reduced, and is stored in pieces (store_row_vector).  Only an
+// element in a half dword that the range check drops at the very end of the buffer needs a
+// 2-byte load of its own.  total = rows * nvr vectors per launch; all byte offsets of a
+// launch stay below 2^31.  Outputs take the default cache policy: rows share cache lines
+// between store instructions, which the L2 merges.
+template <typename T>
+__device__ __forceinline__ Words<4> load_half_row_vector(rsrc_t r, u32 off, u32 rem) {
+    Words<4> v = buf_load<4, kStream>(r, off);
+    if (sizeof(T) == 2 && rem < 16u && (rem & 2u)) {
+        const u32 bits = load_b16<kStream>(r, off + (rem & ~3u));
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if ((u32)j == rem / 4u) v.v[j] = bits;
+    }
+    return v;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_fwd_ragged(T* __restrict__ h, const T* __restrict__ gu, uint32_t rows, uint32_t total, uint32_t half_bytes,
+                  FastDiv nvr, int xcd_group) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const uint32_t v = (uint32_t)xcd_remap(blockIdx.x, gridDim.x, xcd_group) * 256u + threadIdx.x;
+    if (v >= total) return;
+    const rsrc_t rin = make_rsrc(gu, rows * 2u * half_bytes);
+    const rsrc_t rout = make_rsrc(h, rows * half_bytes);
+    const uint32_t row = fastdiv(v, nvr);
+    const uint32_t pos = (v - row * nvr.d) * 16u;
+    const uint32_t rem = half_bytes - pos;
+    const uint32_t gi = row * 2u * half_bytes + pos;
+    const Words<4> g = load_half_row_vector<T>(rin, gi, rem);
+    const Words<4> u = load_half_row_vector<T>(rin, gi + half_bytes, rem);
+    float gf[EPV], uf[EPV], o[EPV];
+    unpack_vec<T, 4>(g, gf);
+    unpack_vec<T, 4>(u, uf);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) o[e] = (gf[e] * fast_sigmoid(gf[e])) * uf[e];
+    store_row_vector<kKeep>(rout, row * half_bytes + pos, rem, pack_vec<T, 4>(o));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+swiglu_bwd_ragged(T* __restrict__ dgu, const T* __restrict__ dh, const T* __restrict__ gu, uint32_t rows,
+                  uint32_t total, uint32_t half_bytes, FastDiv nvr, int xcd_group) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const uint32_t v = (uint32_t)xcd_remap(blockIdx.x, gridDim.x, xcd_group) * 256u + threadIdx.x;
+    if (v >= total) return;
+    const rsrc_t rin = make_rsrc(gu, rows * 2u * half_bytes);
+    const rsrc_t rdh = make_rsrc(dh, rows * half_bytes);
+    const rsrc_t rout = make_rsrc(dgu, rows * 2u * half_bytes);
+    const uint32_t row = fastdiv(v, nvr);
+    const uint32_t pos = (v - row * nvr.d) * 16u;
+    const uint32_t rem = half_bytes - pos;
+    const uint32_t gi = row * 2u * half_bytes + pos;
+    const Words<4> g = load_half_row_vector<T>(rin, gi, rem);
+    const Words<4> u = load_half_row_vector<T>(rin, gi + half_bytes, rem);
+    const Words<4> d = load_half_row_vector<T>(rdh, row * half_bytes + pos, rem);
+    float gf[EPV], uf[EPV], df[EPV], og[EPV], ou[EPV];
+    unpack_vec<T, 4>(g, gf);
+    unpack_vec<T, 4>(u, uf);
+    unpack_vec<T, 4>(d, df);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+        const float sg = fast_sigmoid(gf[e]);
+        ou[e] = df[e] * (gf[e] * sg);
+        og[e] = (df[e] * uf[e]) * (sg * __builtin_fmaf(gf[e], 1.0f - sg, 1.0f));
+    }
+    store_row_vector<kKeep>(rout, gi, rem, pack_vec<T, 4>(og));
+    store_row_vector<kKeep>(rout, gi + half_bytes, rem, pack_vec<T, 4>(ou));
+}
+
+// Element-wise variants, kept for comparison (the "force_generic" option).
 // total = M * H elements (< 2^32 per launch), hdiv divides by H.
 template <typename T>
 __global__ void __launch_bounds__(256)

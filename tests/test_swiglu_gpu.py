@@ -77,6 +77,39 @@ def test_extreme_gates(dtype):
 
 
 @pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("M,H,off", [(301, 1001, 0), (77, 1376, 3), (1000, 100, 1), (19, 7, 0), (4097, 33, 5), (9, 2049, 2)])
+def test_any_width_and_alignment(dtype, M, H, off):
+    """Half rows that are not whole 16-byte vectors (odd widths included) and bases `off`
+    elements away from an aligned address: the 16-byte kernels for ragged rows.  Outputs sit
+    between canary elements that must stay untouched."""
+    td = U.DTYPES[dtype]
+    gu, dh = _inputs(M, H, dtype, seed=M + 3 * H + off, scale=2.0)
+    h_ref, d_ref, floor = U.swiglu_reference(gu, dh, dtype)
+    PAD = 32
+
+    def placed(shape, src=None):
+        n = shape[0] * shape[1]
+        buf = torch.full((PAD + off + n + PAD,), 7.0, dtype=td, device="cuda")
+        view = buf[PAD + off: PAD + off + n].view(*shape)
+        if src is not None:
+            view.copy_(src)
+        return buf, view, n
+
+    _, gud, _ = placed((M, 2 * H), gu)
+    _, dhd, _ = placed((M, H), dh)
+    hbuf, h, hn = placed((M, H))
+    dbuf, d, dn = placed((M, 2 * H))
+    L = U.lib()
+    U.check(L.mg_swiglu_fwd(h.data_ptr(), gud.data_ptr(), M, H, U.CODES[dtype], U.stream()))
+    U.check(L.mg_swiglu_bwd(d.data_ptr(), dhd.data_ptr(), gud.data_ptr(), M, H, U.CODES[dtype], U.stream()))
+    torch.cuda.synchronize()
+    for buf, n in ((hbuf, hn), (dbuf, dn)):
+        assert (buf[:PAD + off] == 7).all() and (buf[PAD + off + n:] == 7).all(), "wrote outside the output"
+    U.assert_matches(h, h_ref, dtype, f"h {M}x{H}+{off}")
+    U.assert_matches(d, d_ref, dtype, f"dgu {M}x{H}+{off}", floor=floor)
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_generic_kernels_match_oracle(dtype):
     M, H = 64, 512
     gu, dh = _inputs(M, H, dtype, seed=77)
@@ -90,7 +123,7 @@ def test_generic_kernels_match_oracle(dtype):
         U.check(U.lib().mg_set_option(b"force_generic", 0))
     U.assert_matches(h, h_ref, dtype, "h (forced generic)")
     U.assert_matches(d, d_ref, dtype, "dgu (forced generic)", floor=floor)
-    # a base pointer that is not 16-byte aligned takes the same path by itself
+    # a base pointer that is not 16-byte aligned takes the any-alignment vector kernels
     pad = torch.empty(M * 2 * H + 1, dtype=U.DTYPES[dtype], device="cuda")
     gm = pad[1:].view(M, 2 * H)
     gm.copy_(gud)
