@@ -114,12 +114,12 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
     return false;
 }
 
-// Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  Measured on MI355X,
-// about 64 KiB of loads in flight per compute unit saturates HBM and more waves than that
-// only add contention, so: the most threads per row (fewest vectors per thread) that still
-// keep (row slots) x (row bytes) x (x and dy) x (current + prefetched row) >= 36 KiB
-// (sweep over 576...10240 columns: two vectors per thread beat three at half the threads by
-// 4-10 %, e.g. 1280 columns 6.3 against 5.7 TB/s, while 4096 columns still want 256 x 2).
+// Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  From sweeps over
+// 576...16384 columns on MI355X: the fewest threads per row that keep a thread at or below
+// two vectors -- three vectors at half the threads lose 4-23 % (1032 columns: 5.0 against
+// 6.1 TB/s, 4104: 5.4 against 6.1), and one vector at twice the threads loses at the
+// 4096 x 4096 shape (20.5 against 18.9 us).  Rows of more than 1024 vectors take what fits:
+// 512 x 3, 1024 x 2, 512 x 4...8.
 bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
@@ -139,15 +139,12 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         return true;
     }
     for (int b : {block == 1024 ? 1024 : 512, 512}) {
-        for (int t = b; t >= 64; t /= 2) {
-            const int need = round_items(ceil_div(nvec, t));
-            const long in_flight = (long)(b / t) * row_bytes * 4;
-            if (in_flight >= 36 * 1024 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
+        for (int t = 64; t <= b; t *= 2) {
+            const int need = ceil_div(nvec, t);
+            if (need <= 2 && bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
         }
-        for (int t = 64; t <= b; t *= 2) {  // short rows: as many row slots as the workgroup has waves
-            const int need = round_items(ceil_div(nvec, t));
-            if (bwd_cfg_ok(esize, t, need, b)) { *cfg = {kVec, t, need, b}; return true; }
-        }
+        const int need = round_items(ceil_div(nvec, b));   // wider than two vectors per thread of a workgroup
+        if (bwd_cfg_ok(esize, b, need, b)) { *cfg = {kVec, b, need, b}; return true; }
     }
     return false;
 }

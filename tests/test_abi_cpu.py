@@ -141,11 +141,11 @@ def _launch_info(lib, backward, cols, dtype):
     # 2-byte types: 8 elements per 16-byte vector
     (4096, 2, (0, 256, 2, 256), (0, 256, 2, 512)),      # metric shape: one row per 256-thread workgroup
     (2048, 1, (0, 128, 2, 256), (0, 128, 2, 512)),
-    (4100, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
+    (4100, 2, (0, 256, 3, 256), (0, 512, 2, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
     (5120, 1, (0, 512, 2, 512), (0, 512, 2, 512)),
     (8192, 2, (0, 512, 2, 512), (0, 512, 2, 512)),
     (16384, 2, (0, 1024, 2, 1024), (0, 1024, 2, 1024)),
-    (4099, 2, (0, 256, 3, 256), (0, 256, 3, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
+    (4099, 2, (0, 256, 3, 256), (0, 512, 2, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # wider than registers hold
     # rows of up to 2 KiB share a wave: 8, 16 or 32 lanes per row;
     # forward up to 4 vectors per lane (128 vectors), backward up to 2 (56 vectors)
@@ -157,7 +157,7 @@ def _launch_info(lib, backward, cols, dtype):
     (512, 2, (0, 16, 4, 256), (0, 64, 1, 512)),         # 64 vectors: backward takes one wave per row
     (768, 2, (0, 32, 3, 256), (0, 64, 2, 512)),
     (1024, 1, (0, 32, 4, 256), (0, 64, 2, 512)),
-    (1032, 2, (0, 64, 3, 256), (0, 64, 3, 512)),        # 129 vectors: one wave per row
+    (1032, 2, (0, 64, 3, 256), (0, 128, 2, 512)),        # 129 vectors: one wave per row
     (100, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # pitch 200 bytes: the last vector of a row is trimmed
     (299, 1, (0, 16, 3, 256), (0, 16, 3, 512)),         # 598 bytes, rows only 2-byte aligned
     (999, 1, (0, 64, 2, 256), (0, 64, 2, 512)),         # 1998 bytes: too long for that to pay
