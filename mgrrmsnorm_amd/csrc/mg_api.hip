@@ -93,7 +93,7 @@ int round_items(int items) { return (items == 5 || items == 7) ? items + 1 : ite
 bool choose_fwd(long row_bytes, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_fwd_tpr.load(), items = opt_fwd_items.load();
-    {   // rows narrower than a wave: several rows per wave (a requested 8 or 16 wins when it fits)
+    {   // rows narrower than a wave: several rows per wave (a requested 8, 16 or 32 wins when it fits)
         const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes, false) : 0);
         if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 0}; return true; }
     }

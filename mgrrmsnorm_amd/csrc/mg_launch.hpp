@@ -9,7 +9,7 @@ namespace mg {
 // How a row is spread over threads in the register-resident RMSNorm kernels.
 struct RowCfg {
     int vec;    // bytes per vector load (16)
-    int tpr;    // threads per row: 64, 128, 256, 512, 1024; 8 or 16 = several rows per wave
+    int tpr;    // threads per row: 64, 128, 256, 512, 1024; 8, 16 or 32 = several rows per wave
     int items;  // vectors per thread
     int block;  // backward only: threads per workgroup, 1024 or 512
 };
