@@ -139,7 +139,9 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
  * takes for rows of `cols` elements; no counterpart in
  * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
  * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
- * workgroup per row, *vectors_per_thread = 0).  *threads_per_row below 64 means that
+ * workgroup per row, *vectors_per_thread = 0).  *generic = 0 with *vectors_per_thread = 0
+ * means a row too wide for registers, streamed twice by a 1024-thread workgroup.
+ * *threads_per_row below 64 means that
  * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
  * 640 bytes when the pitch is not a multiple of 16 bytes).
  */

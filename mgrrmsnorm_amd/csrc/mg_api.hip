@@ -149,11 +149,19 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     return false;
 }
 
+// Rows that no register-resident shape holds: 1024 threads stream the row twice
+// (vectors_per_thread = 0 in the launch report: it is not fixed).
+bool choose_streaming(long row_bytes, RowCfg* cfg) {
+    if (!streaming_ok(row_bytes)) return false;
+    *cfg = {kVec, 1024, 0, 1024, kFamilyStreaming};
+    return true;
+}
+
 // Requesting row i+1 before reducing row i doubles the bytes a workgroup keeps in flight; it
 // pays up to about 80 KiB (x and dy, current and next row, all row slots) and costs
 // throughput beyond (12288 bf16 columns: 5.75 TB/s with, 6.09 without).
 bool bwd_prefetch_default(const RowCfg& cfg, long row_bytes) {
-    if (narrow_tpr(cfg.tpr) || cfg.tpr <= 0) return true;
+    if (narrow_tpr(cfg.tpr) || cfg.tpr <= 0 || cfg.family != kFamilyResident) return true;
     return (long)(cfg.block / cfg.tpr) * row_bytes * 4 <= 80 * 1024;
 }
 
@@ -219,7 +227,7 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) generic = !choose_fwd(row_bytes, &cfg);
+    if (!generic) generic = !choose_fwd(row_bytes, &cfg) && !choose_streaming(row_bytes, &cfg);
     const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps, xcd_group_or(kXcdGroupStreaming)};
     hipStream_t s = (hipStream_t)stream;
     hipError_t e = by_dtype(
@@ -241,11 +249,12 @@ int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, 
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool gen = opt_force_generic.load() != 0;
-    if (!gen) gen = backward ? !choose_bwd(row_bytes, es, &cfg) : !choose_fwd(row_bytes, &cfg);
+    if (!gen) gen = !(backward ? choose_bwd(row_bytes, es, &cfg) : choose_fwd(row_bytes, &cfg)) &&
+                    !choose_streaming(row_bytes, &cfg);
     *generic = gen ? 1 : 0;
     *threads_per_row = gen ? 256 : cfg.tpr;
     *vectors_per_thread = gen ? 0 : cfg.items;
-    *workgroup_threads = gen ? 256 : (backward ? cfg.block : (cfg.tpr > 256 ? cfg.tpr : 256));
+    *workgroup_threads = gen ? 256 : (backward || cfg.family == kFamilyStreaming ? cfg.block : (cfg.tpr > 256 ? cfg.tpr : 256));
     return MG_OK;
 }
 
@@ -311,7 +320,7 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) generic = !choose_bwd(row_bytes, es, &cfg);
+    if (!generic) generic = !choose_bwd(row_bytes, es, &cfg) && !choose_streaming(row_bytes, &cfg);
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,

@@ -12,7 +12,12 @@ struct RowCfg {
     int tpr;    // threads per row: 64, 128, 256, 512, 1024; 8, 16 or 32 = several rows per wave
     int items;  // vectors per thread
     int block;  // backward only: threads per workgroup, 1024 or 512
+    int family; // kFamilyResident (rows held in registers) or kFamilyStreaming (rows read twice)
 };
+constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
+// Rows that do not fit registers stream through 1024-thread workgroups when their pitch is
+// a multiple of 4 bytes (no half dword at the end of a row).
+constexpr bool streaming_ok(long row_bytes) { return row_bytes % 4 == 0; }
 
 constexpr int kVec = 16;
 

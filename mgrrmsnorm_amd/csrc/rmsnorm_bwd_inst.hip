@@ -95,6 +95,18 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
                 a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
         return hipGetLastError();
     }
+    if (cfg.family == kFamilyStreaming) {
+        rmsnorm_bwd_dx_wide<elem_t><<<dim3((unsigned)a.rows), dim3(kWideBlock), 0, s>>>(
+            (elem_t*)a.dx, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows, a.cols,
+            1.0f / (float)a.cols);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const long nvec = ((long)a.cols * (long)sizeof(elem_t) + kVec - 1) / kVec;
+        rmsnorm_bwd_dw_wide<elem_t>
+            <<<dim3((unsigned)((nvec + 255) / 256), (unsigned)a.num_partials), dim3(256), 0, s>>>(
+                a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
+        return hipGetLastError();
+    }
     if (cfg.vec != kVec) return hipErrorInvalidValue;
     if (cfg.tpr == 8 && cfg.block == 512) return narrow_by_items<8>(cfg.items, a, s);
     if (cfg.tpr == 16 && cfg.block == 512) return narrow_by_items<16>(cfg.items, a, s);

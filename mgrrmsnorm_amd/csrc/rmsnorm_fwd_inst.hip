@@ -91,6 +91,12 @@ hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const Fwd
             1.0f / (float)a.cols);
         return hipGetLastError();
     }
+    if (cfg.family == kFamilyStreaming) {
+        rmsnorm_fwd_wide<elem_t><<<dim3((unsigned)a.rows), dim3(kWideBlock), 0, s>>>(
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+            1.0f / (float)a.cols);
+        return hipGetLastError();
+    }
     if (cfg.vec == kVec) return by_tpr<kVec>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;
 }

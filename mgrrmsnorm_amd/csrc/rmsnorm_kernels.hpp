@@ -600,6 +600,181 @@ rmsnorm_bwd_dw_generic(float* __restrict__ dw_part, int ld, const T* __restrict_
 }
 
 // =================================================================================
+// Rows too wide for registers (row pitch a multiple of 4 bytes): one 1024-thread workgroup
+// per row streams the row twice with 16-byte buffer accesses -- once for the row sum, once
+// for the output; the second read of a row that fits the L2 comes from there.  Four vectors
+// per thread are in flight at a time; offsets past the row load 0 and store nothing.
+// =================================================================================
+constexpr int kWideBlock = 1024;
+constexpr int kWideInFlight = 4;
+
+// Sum over the 1024 threads of a workgroup, identical in every thread: DPP inside the waves,
+// then the 16 wave sums through LDS in wave order.
+__device__ __forceinline__ float wide_block_sum(float v, float* lds16) {
+    v = wave_sum(v);
+    __syncthreads();   // lds16 may still be read from a previous sum
+    if ((threadIdx.x & (kWave - 1)) == 0) lds16[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float t = 0.0f;
+#pragma unroll
+    for (int k = 0; k < kWideBlock / kWave; ++k) t += lds16[k];
+    return t;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kWideBlock)
+rmsnorm_fwd_wide(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                 const T* __restrict__ w, long rows, int cols, float eps, float inv_cols) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    __shared__ float lds16[kWideBlock / kWave];
+    const long row = blockIdx.x;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = (row_bytes + 15u) / 16u;
+    const rsrc_t rx = make_rsrc(x + row * (long)cols, row_bytes);
+    const rsrc_t ry = make_rsrc(y + row * (long)cols, row_bytes);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+    const u32 stride = kWideBlock * kWideInFlight;
+
+    float ss = 0.0f;
+    for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
+        Words<4> xv[kWideInFlight];
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) xv[k] = buf_load<4, kKeep>(rx, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) {
+            float f[EPV];
+            unpack_vec<T, 4>(xv[k], f);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) ss = __builtin_fmaf(f[e], f[e], ss);
+        }
+    }
+    ss = wide_block_sum(ss, lds16);
+    const float s = fast_rsqrt(ss * inv_cols + eps);
+    if (threadIdx.x == 0 && inv_rms != nullptr) inv_rms[row] = s;
+
+    for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
+        Words<4> xv[kWideInFlight], wv[kWideInFlight];
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) xv[k] = buf_load<4, kStream>(rx, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) wv[k] = buf_load<4, kKeep>(rw, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) {
+            float xf[EPV], wf[EPV], o[EPV];
+            unpack_vec<T, 4>(xv[k], xf);
+            unpack_vec<T, 4>(wv[k], wf);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) o[e] = (xf[e] * s) * wf[e];
+            buf_store<4, kStream>(ry, (v0 + k * kWideBlock) * 16u, pack_vec<T, 4>(o));
+        }
+    }
+}
+
+// dx for rows too wide for registers: pass 1 sums dy*w*x over the row, pass 2 writes dx.
+template <typename T>
+__global__ void __launch_bounds__(kWideBlock)
+rmsnorm_bwd_dx_wide(T* __restrict__ dx, const T* __restrict__ dy, const T* __restrict__ x,
+                    const T* __restrict__ w, const float* __restrict__ inv_rms, long rows, int cols,
+                    float inv_cols) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    __shared__ float lds16[kWideBlock / kWave];
+    const long row = blockIdx.x;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = (row_bytes + 15u) / 16u;
+    const rsrc_t rx = make_rsrc(x + row * (long)cols, row_bytes);
+    const rsrc_t rg = make_rsrc(dy + row * (long)cols, row_bytes);
+    const rsrc_t rd = make_rsrc(dx + row * (long)cols, row_bytes);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+    const u32 stride = kWideBlock * kWideInFlight;
+    const float s = inv_rms[row];
+
+    float a = 0.0f;
+    for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
+        Words<4> xv[kWideInFlight], gv[kWideInFlight], wv[kWideInFlight];
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) xv[k] = buf_load<4, kKeep>(rx, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) gv[k] = buf_load<4, kKeep>(rg, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) wv[k] = buf_load<4, kKeep>(rw, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) {
+            float xf[EPV], gf[EPV], wf[EPV];
+            unpack_vec<T, 4>(xv[k], xf);
+            unpack_vec<T, 4>(gv[k], gf);
+            unpack_vec<T, 4>(wv[k], wf);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) a = __builtin_fmaf(gf[e] * xf[e], wf[e], a);
+        }
+    }
+    a = wide_block_sum(a, lds16);
+    const float c2 = a * (s * s) * s * inv_cols;
+
+    for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
+        Words<4> xv[kWideInFlight], gv[kWideInFlight], wv[kWideInFlight];
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) xv[k] = buf_load<4, kStream>(rx, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) gv[k] = buf_load<4, kStream>(rg, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) wv[k] = buf_load<4, kKeep>(rw, (v0 + k * kWideBlock) * 16u);
+#pragma unroll
+        for (int k = 0; k < kWideInFlight; ++k) {
+            float xf[EPV], gf[EPV], wf[EPV], o[EPV];
+            unpack_vec<T, 4>(xv[k], xf);
+            unpack_vec<T, 4>(gv[k], gf);
+            unpack_vec<T, 4>(wv[k], wf);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) o[e] = __builtin_fmaf(gf[e] * wf[e], s, -(xf[e] * c2));
+            buf_store<4, kStream>(rd, (v0 + k * kWideBlock) * 16u, pack_vec<T, 4>(o));
+        }
+    }
+}
+
+// dW partials for rows too wide for registers: grid = (ceil(nvec / 256), P); a thread owns
+// one 16-byte vector of columns and the rows p, p + P, p + 2P, ... (four rows in flight).
+template <typename T>
+__global__ void __launch_bounds__(256)
+rmsnorm_bwd_dw_wide(float* __restrict__ dw_part, int ld, const T* __restrict__ dy, const T* __restrict__ x,
+                    const float* __restrict__ inv_rms, long rows, int cols) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 vec = blockIdx.x * 256u + threadIdx.x;
+    const u32 off = vec * 16u;          // past the row for the lanes beyond it: loads 0
+    const long p = blockIdx.y, P = gridDim.y;
+    float acc[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) acc[e] = 0.0f;
+    for (long r0 = p; r0 < rows; r0 += 4 * P) {
+        Words<4> xv[4], gv[4];
+        float sr[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const long r = r0 + k * P;
+            const bool live = r < rows;
+            const long base = live ? r * (long)cols : 0;
+            xv[k] = buf_load<4, kStream>(make_rsrc(x + base, live ? row_bytes : 0u), off);
+            gv[k] = buf_load<4, kStream>(make_rsrc(dy + base, live ? row_bytes : 0u), off);
+            sr[k] = live ? inv_rms[r] : 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            float xf[EPV], gf[EPV];
+            unpack_vec<T, 4>(xv[k], xf);
+            unpack_vec<T, 4>(gv[k], gf);
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) acc[e] = __builtin_fmaf(gf[e] * xf[e], sr[k], acc[e]);
+        }
+    }
+    float* out = dw_part + p * (long)ld;
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) {
+        const long c = (long)vec * EPV + e;
+        if (c < ld) out[c] = acc[e];
+    }
+}
+
+// =================================================================================
 // Backward pass 2: dW[c] = sum_p part[p, c] in a fixed order.
 //   block = 256 threads = 8 column quads (32 columns = one 128-byte line per partial row)
 //   x 32 row subsets; thread (q, sub) adds rows sub, sub+32, ... with eight independent

@@ -60,6 +60,9 @@ SHAPES = [
     (3, 33000),      # wider than the register-resident kernels hold for 2-byte types
     (1000, 12),
     (2, 65536),      # the widest row the forward register-resident kernels hold for 2-byte types
+    (5, 70000),      # beyond that: rows streamed twice by 1024-thread workgroups (forward and backward)
+    (3, 70001),      # ... and one element per thread when such a row ends in half a dword
+    (300, 40002),    # backward streams (two launches: dx, dW partials), forward holds the row
     # rows narrower than a wave (pitch a multiple of 16 bytes): several rows share a wave
     (1000, 64),      # 8 lanes per row for 2-byte types; 1000 = 125 full waves of 8 rows
     (1003, 128),     # the last wave holds 3 rows of its 8
