@@ -14,8 +14,11 @@
 // Narrow family: rows of at most 128 vectors put 8, 16 or 32 lanes on a row, so that one
 // wave carries 8, 4 or 2 consecutive rows (see below).
 //
+// Streaming family: rows that do not fit registers are read twice by one 1024-thread
+// workgroup per row, with the same 16-byte accesses.
+//
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
-// the row; used when the row does not fit the register-resident family (or on request).
+// the row; used on request, and for rows beyond registers that end in half a dword.
 #pragma once
 #include "mg_device.hpp"
 
