@@ -163,7 +163,7 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
  * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
  * the current one; -1 = automatic), "swiglu_unroll",
- * "force_generic" (1 = always take the unvectorised path), "xcd_group" (consecutive workgroups
+ * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
  * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
  * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for
  * an unknown key.  Values that do not fit a given problem are ignored for that call.

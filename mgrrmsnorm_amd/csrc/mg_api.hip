@@ -152,7 +152,7 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
 // Rows that no register-resident shape holds: 1024 threads stream the row twice
 // (vectors_per_thread = 0 in the launch report: it is not fixed).
 bool choose_streaming(long row_bytes, RowCfg* cfg) {
-    if (!streaming_ok(row_bytes)) return false;
+    (void)row_bytes;
     *cfg = {kVec, 1024, 0, 1024, kFamilyStreaming};
     return true;
 }

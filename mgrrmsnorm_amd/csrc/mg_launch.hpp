@@ -15,9 +15,7 @@ struct RowCfg {
     int family; // kFamilyResident (rows held in registers) or kFamilyStreaming (rows read twice)
 };
 constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
-// Rows that do not fit registers stream through 1024-thread workgroups when their pitch is
-// a multiple of 4 bytes (no half dword at the end of a row).
-constexpr bool streaming_ok(long row_bytes) { return row_bytes % 4 == 0; }
+// Rows that do not fit registers stream through 1024-thread workgroups.
 
 constexpr int kVec = 16;
 

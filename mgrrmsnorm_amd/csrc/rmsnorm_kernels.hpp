@@ -603,7 +603,7 @@ rmsnorm_bwd_dw_generic(float* __restrict__ dw_part, int ld, const T* __restrict_
 }
 
 // =================================================================================
-// Rows too wide for registers (row pitch a multiple of 4 bytes): one 1024-thread workgroup
+// Rows too wide for registers: one 1024-thread workgroup
 // per row streams the row twice with 16-byte buffer accesses -- once for the row sum, once
 // for the output; the second read of a row that fits the L2 comes from there.  Four vectors
 // per thread are in flight at a time; offsets past the row load 0 and store nothing.
@@ -651,9 +651,18 @@ rmsnorm_fwd_wide(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
             for (int e = 0; e < EPV; ++e) ss = __builtin_fmaf(f[e], f[e], ss);
         }
     }
+    // a row of an odd number of 2-byte elements ends in half a dword, which the range check
+    // drops from the vectors: thread 0 carries that element by itself
+    const bool odd_tail = sizeof(T) == 2 && (row_bytes & 2u) != 0 && threadIdx.x == 0;
+    float x_last = 0.0f;
+    if (odd_tail) {
+        x_last = Elem<T>::load1(x + row * (long)cols + (cols - 1));
+        ss = __builtin_fmaf(x_last, x_last, ss);
+    }
     ss = wide_block_sum(ss, lds16);
     const float s = fast_rsqrt(ss * inv_cols + eps);
     if (threadIdx.x == 0 && inv_rms != nullptr) inv_rms[row] = s;
+    if (odd_tail) Elem<T>::store1(y + row * (long)cols + (cols - 1), (x_last * s) * Elem<T>::load1(w + (cols - 1)));
 
     for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
         Words<4> xv[kWideInFlight], wv[kWideInFlight];
@@ -710,8 +719,18 @@ rmsnorm_bwd_dx_wide(T* __restrict__ dx, const T* __restrict__ dy, const T* __res
             for (int e = 0; e < EPV; ++e) a = __builtin_fmaf(gf[e] * xf[e], wf[e], a);
         }
     }
+    // the element in the half dword that ends a row of an odd number of 2-byte elements
+    const bool odd_tail = sizeof(T) == 2 && (row_bytes & 2u) != 0 && threadIdx.x == 0;
+    float x_last = 0.0f, gw_last = 0.0f;
+    if (odd_tail) {
+        const long at = row * (long)cols + (cols - 1);
+        x_last = Elem<T>::load1(x + at);
+        gw_last = Elem<T>::load1(dy + at) * Elem<T>::load1(w + (cols - 1));
+        a = __builtin_fmaf(gw_last, x_last, a);
+    }
     a = wide_block_sum(a, lds16);
     const float c2 = a * (s * s) * s * inv_cols;
+    if (odd_tail) Elem<T>::store1(dx + row * (long)cols + (cols - 1), __builtin_fmaf(gw_last, s, -(x_last * c2)));
 
     for (u32 v0 = threadIdx.x; v0 < nvec; v0 += stride) {
         Words<4> xv[kWideInFlight], gv[kWideInFlight], wv[kWideInFlight];
@@ -745,6 +764,10 @@ rmsnorm_bwd_dw_wide(float* __restrict__ dw_part, int ld, const T* __restrict__ d
     const u32 vec = blockIdx.x * 256u + threadIdx.x;
     const u32 off = vec * 16u;          // past the row for the lanes beyond it: loads 0
     const long p = blockIdx.y, P = gridDim.y;
+    // the thread whose vector holds the half dword that ends an odd row of 2-byte elements
+    // fetches that element with 2-byte loads and puts it where the vector load left 0
+    const bool odd_tail = sizeof(T) == 2 && (row_bytes & 2u) != 0 && vec == (row_bytes - 1u) / 16u;
+    const int tail_word = (int)(((row_bytes - 2u) % 16u) / 4u);
     float acc[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) acc[e] = 0.0f;
@@ -756,8 +779,16 @@ rmsnorm_bwd_dw_wide(float* __restrict__ dw_part, int ld, const T* __restrict__ d
             const long r = r0 + k * P;
             const bool live = r < rows;
             const long base = live ? r * (long)cols : 0;
-            xv[k] = buf_load<4, kStream>(make_rsrc(x + base, live ? row_bytes : 0u), off);
-            gv[k] = buf_load<4, kStream>(make_rsrc(dy + base, live ? row_bytes : 0u), off);
+            const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
+            const rsrc_t rg = make_rsrc(dy + base, live ? row_bytes : 0u);
+            xv[k] = buf_load<4, kStream>(rx, off);
+            gv[k] = buf_load<4, kStream>(rg, off);
+            if (odd_tail) {
+                const u32 xb = load_b16<kStream>(rx, row_bytes - 2u), gb = load_b16<kStream>(rg, row_bytes - 2u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (j == tail_word) { xv[k].v[j] = xb; gv[k].v[j] = gb; }
+            }
             sr[k] = live ? inv_rms[r] : 0.0f;
         }
 #pragma unroll

@@ -147,7 +147,7 @@ def _launch_info(lib, backward, cols, dtype):
     (16384, 2, (0, 1024, 2, 1024), (0, 1024, 2, 1024)),
     (4099, 2, (0, 256, 3, 256), (0, 512, 2, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # wider than registers hold: 1024 threads stream the row twice
-    (100001, 1, (1, 256, 0, 256), (1, 256, 0, 256)),    # ... and an odd width of a 2-byte type: one element per thread
+    (100001, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # ... an odd width of a 2-byte type too
     (40000, 2, (0, 1024, 5, 1024), (0, 1024, 0, 1024)),   # the backward pass holds fewer vectors than the forward pass
     # rows of up to 2 KiB share a wave: 8, 16 or 32 lanes per row;
     # forward up to 4 vectors per lane (128 vectors), backward up to 2 (56 vectors)

@@ -61,7 +61,8 @@ SHAPES = [
     (1000, 12),
     (2, 65536),      # the widest row the forward register-resident kernels hold for 2-byte types
     (5, 70000),      # beyond that: rows streamed twice by 1024-thread workgroups (forward and backward)
-    (3, 70001),      # ... and one element per thread when such a row ends in half a dword
+    (3, 70001),      # ... also when such a row ends in half a dword (2-byte types)
+    (70, 33001),     # backward streams an odd width; 70 rows exceed the four rows a dW thread has in flight
     (300, 40002),    # backward streams (two launches: dx, dW partials), forward holds the row
     # rows narrower than a wave (pitch a multiple of 16 bytes): several rows share a wave
     (1000, 64),      # 8 lanes per row for 2-byte types; 1000 = 125 full waves of 8 rows
