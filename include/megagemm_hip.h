@@ -114,6 +114,26 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
                          int64_t num_partials, int64_t ld, int64_t cols, void* stream);
 
 /*
+ * RMSNorm backward for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  It does what mg_rmsnorm_bwd followed by mg_rmsnorm_dw_reduce does -- dx, and dW
+ * as dw_f32 ([cols] fp32) and/or dw_cast ([cols] of `dtype`); at least one of the two -- but
+ * keeps the dW partials in a device array of MG_NOALLOC_SCRATCH_BYTES that belongs to the
+ * library (one copy per GPU the library runs on, held until the process ends) instead of a
+ * workspace of the caller's.  It calls no allocating routine.  The number of partial rows is
+ * the one mg_rmsnorm_bwd_workspace reports, capped at MG_NOALLOC_SCRATCH_BYTES / (4 * ld);
+ * results are bit-identical to the two-call sequence with that number of partial rows.
+ * cols above MG_NOALLOC_MAX_COLS is rejected with MG_ERR_UNSUPPORTED.
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it; calls ordered by a stream or by events do not.
+ */
+#define MG_NOALLOC_SCRATCH_BYTES (16 << 20)
+#define MG_NOALLOC_MAX_COLS 65536
+int mg_rmsnorm_bwd_noalloc(void* dx, float* dw_f32, void* dw_cast, const void* dy, const void* x,
+                           const void* w, const float* inv_rms, int64_t rows, int64_t cols, int dtype,
+                           void* stream);
+
+/*
  * SwiGLU activation forward.  Replaces the launch of _mg_swiglu_fwd_kernel
  * (megagemm/swiglu.py:18-43, launch :100-107).
  *

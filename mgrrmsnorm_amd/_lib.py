@@ -37,6 +37,7 @@ SIGNATURES = {
     "mg_rmsnorm_bwd_workspace": (_int, [_i64, _i64, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64)]),
     "mg_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _i64, _vp]),
     "mg_rmsnorm_dw_reduce": (_int, [_vp, _vp, _int, _vp, _i64, _i64, _i64, _vp]),
+    "mg_rmsnorm_bwd_noalloc": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mg_swiglu_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mg_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mg_copy_bytes": (_int, [_vp, _vp, _i64, _vp]),

@@ -358,6 +358,54 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
     return MG_OK;
 }
 
+// ---- the entry point that allocates nothing ----
+// dW partials live in a device array of the library itself.  The array's name is a host-side
+// handle, not a device address: its per-device address is fetched once with
+// hipGetSymbolAddress and that pointer is what the kernels get.
+constexpr int64_t kScratchFloats = (int64_t)MG_NOALLOC_SCRATCH_BYTES / 4;
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+static int scratch_address(float** out) {
+    static std::atomic<float*> cache[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd_noalloc: hipGetDevice", e);
+    if (dev >= 0 && dev < 64) {
+        float* p = cache[dev].load(std::memory_order_acquire);
+        if (p != nullptr) { *out = p; return MG_OK; }
+    }
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || addr == nullptr)
+        return fail_hip("mg_rmsnorm_bwd_noalloc: hipGetSymbolAddress(scratch)", e == hipSuccess ? hipErrorInvalidSymbol : e);
+    if (dev >= 0 && dev < 64) cache[dev].store((float*)addr, std::memory_order_release);
+    *out = (float*)addr;
+    return MG_OK;
+}
+
+int mg_rmsnorm_bwd_noalloc(void* dx, float* dw_f32, void* dw_cast, const void* dy, const void* x, const void* w,
+                           const float* inv_rms, int64_t rows, int64_t cols, int dtype, void* stream) {
+    int rc = check_rmsnorm_dims("mg_rmsnorm_bwd_noalloc", rows, cols, dtype);
+    if (rc != MG_OK) return rc;
+    if (cols > MG_NOALLOC_MAX_COLS)
+        return fail(MG_ERR_UNSUPPORTED,
+                    "mg_rmsnorm_bwd_noalloc: cols = %lld is beyond this entry point's maximum of %d; use "
+                    "mg_rmsnorm_bwd with a workspace of the caller's",
+                    (long long)cols, MG_NOALLOC_MAX_COLS);
+    if (dw_f32 == nullptr && dw_cast == nullptr)
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd_noalloc: give dw_f32, dw_cast or both");
+    int64_t num_partials = 0, ld = 0;
+    rc = mg_rmsnorm_bwd_workspace(rows, cols, dtype, &num_partials, &ld);
+    if (rc != MG_OK) return rc;
+    if (num_partials * ld > kScratchFloats) num_partials = kScratchFloats / ld;   // >= 64 rows: ld <= 65536
+    float* part = nullptr;
+    rc = scratch_address(&part);
+    if (rc != MG_OK) return rc;
+    rc = mg_rmsnorm_bwd(dx, part, dy, x, w, inv_rms, rows, cols, dtype, num_partials, ld, stream);
+    if (rc != MG_OK) return rc;
+    return mg_rmsnorm_dw_reduce(dw_f32, dw_cast, dtype, part, num_partials, ld, cols, stream);
+}
+
 int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream) {
     if (bytes < 0 || bytes % 16 != 0 || bytes >= (1LL << 40))
         return fail(MG_ERR_INVALID_ARG, "mg_copy_bytes: bytes must be a non-negative multiple of 16 below 2^40 (got %lld)",

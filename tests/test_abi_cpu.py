@@ -31,7 +31,7 @@ def _declared_functions():
 def test_header_declares_the_expected_entry_points():
     assert _declared_functions() == sorted([
         "mg_abi_version", "mg_last_error", "mg_set_option", "mg_rmsnorm_fwd", "mg_rmsnorm_bwd_workspace",
-        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_swiglu_fwd", "mg_swiglu_bwd", "mg_copy_bytes",
+        "mg_rmsnorm_bwd", "mg_rmsnorm_dw_reduce", "mg_rmsnorm_bwd_noalloc", "mg_swiglu_fwd", "mg_swiglu_bwd", "mg_copy_bytes",
         "mg_rmsnorm_launch_info"])
 
 
