@@ -78,9 +78,11 @@ class RmsNormWorkload:
         self.kernels = {"rmsnorm_fwd": self.fwd_bytes}
         if backward:
             self.kernels["rmsnorm_bwd"] = self.bwd_bytes
+            self.extra_kernels = ["rmsnorm_dw_reduce"]   # timed and reported, bytes belong to rmsnorm_bwd
         self.dominant = "rmsnorm_bwd" if backward else "rmsnorm_fwd"
         self.name = f"rmsnorm_{'fwd_bwd' if backward else 'fwd'}_{rows}x{cols}_{dtype}"
         self.desc = {"rows": rows, "cols": cols, "eps": 1e-6, "launches_per_step": 3 if backward else 1}
+        self.tensor_bytes = rows * cols * e
 
     def _chk(self, rc):
         if rc != 0:
@@ -91,7 +93,7 @@ class RmsNormWorkload:
         self._chk(self.lib.mg_rmsnorm_fwd(s["y"].data_ptr(), s["inv_rms"].data_ptr(), s["x"].data_ptr(),
                                           self.w.data_ptr(), self.rows, self.cols, 1e-6, CODE[self.dtype], st))
 
-    def bwd(self, i, st):
+    def bwd_pass1(self, i, st):
         s = self.sets[i % self.nsets]
         self._chk(self.lib.mg_rmsnorm_bwd(s["dx"].data_ptr(), self.partial.data_ptr(), s["dy"].data_ptr(),
                                           s["x"].data_ptr(), self.w.data_ptr(), s["inv_rms"].data_ptr(), self.rows,
@@ -101,14 +103,27 @@ class RmsNormWorkload:
         self._chk(self.lib.mg_rmsnorm_dw_reduce(self.dw.data_ptr(), None, 0, self.partial.data_ptr(), self.P,
                                                 self.ld, self.cols, st))
 
+    def bwd(self, i, st):
+        """dx and dW: backward pass 1 followed by the dW reduction."""
+        self.bwd_pass1(i, st)
+        self.reduce(i, st)
+
     def step(self, i, st):
         self.fwd(i, st)
         if self.backward:
             self.bwd(i, st)
-            self.reduce(i, st)
 
     def kernel(self, name):
-        return {"rmsnorm_fwd": self.fwd, "rmsnorm_bwd": self.bwd}[name]
+        return {"rmsnorm_fwd": self.fwd, "rmsnorm_bwd": self.bwd_pass1, "rmsnorm_dw_reduce": self.reduce}[name]
+
+    def probe(self, kind, i, st):
+        """Plain streaming launches over this workload's own tensors: the ceiling."""
+        s = self.sets[i % self.nsets]
+        if kind == "copy":      # the forward pass's mix: one read, one write
+            rc = self.lib.mg_stream_probe(s["y"].data_ptr(), s["x"].data_ptr(), None, self.tensor_bytes, st)
+        else:                   # the backward pass's mix: two reads, one write
+            rc = self.lib.mg_stream_probe(s["dx"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), self.tensor_bytes, st)
+        self._chk(rc)
 
 
 class SwigluWorkload:
@@ -134,6 +149,7 @@ class SwigluWorkload:
         self.dominant = "swiglu_bwd"
         self.name = f"swiglu_fwd_bwd_{M}x{H}_{dtype}"
         self.desc = {"M": M, "H": H, "launches_per_step": 2}
+        self.tensor_bytes = M * H * e
 
     def _chk(self, rc):
         if rc != 0:
@@ -155,11 +171,20 @@ class SwigluWorkload:
     def kernel(self, name):
         return {"swiglu_fwd": self.fwd, "swiglu_bwd": self.bwd}[name]
 
+    def probe(self, kind, i, st):
+        s = self.sets[i % self.nsets]
+        if kind == "copy":
+            rc = self.lib.mg_stream_probe(s["h"].data_ptr(), s["dh"].data_ptr(), None, self.tensor_bytes, st)
+        else:
+            rc = self.lib.mg_stream_probe(s["h"].data_ptr(), s["gu"].data_ptr(), s["dh"].data_ptr(), self.tensor_bytes, st)
+        self._chk(rc)
+
 
 def make_workload(lib, name, nsets=0):
     m = re.fullmatch(r"rmsnorm_(fwd_bwd|fwd)_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
     if m:
-        return RmsNormWorkload(lib, int(m.group(2)), int(m.group(3)), m.group(4), backward=m.group(1) == "fwd_bwd", nsets=nsets)
+        return RmsNormWorkload(lib, int(m.group(2)), int(m.group(3)), m.group(4), backward=m.group(1) == "fwd_bwd",
+                               nsets=nsets)
     m = re.fullmatch(r"swiglu_fwd_bwd_(\d+)x(\d+)_(fp32|fp16|bf16)", name)
     if m:
         return SwigluWorkload(lib, int(m.group(1)), int(m.group(2)), m.group(3), nsets=nsets)
@@ -198,10 +223,10 @@ def time_steps(wl, steps, warmup, launch):
     return time.perf_counter() - t0
 
 
-def time_kernel(wl, name, launches=200):
+def time_kernel(wl, name, launches=200, fn=None):
     """Average duration of one launch of `name`, from HIP events around `launches`
     back-to-back launches on the launch stream (buffers rotating). Returns seconds."""
-    fn = wl.kernel(name)
+    fn = fn or wl.kernel(name)
     st = stream_ptr()
     for i in range(10):
         fn(i, st)
@@ -220,14 +245,121 @@ def time_kernel(wl, name, launches=200):
 
 
 def committed_traffic(kernel, workload):
-    """HBM bytes per launch from the committed rocprofv3 counter summary, if there is one."""
+    """HBM bytes per launch from the committed rocprofv3 counter summary (FETCH_SIZE +
+    WRITE_SIZE, calibrated), and where that figure comes from.  It is a counter reading of an
+    earlier profiler run of the same command, not of this run."""
     path = ROOT / "profiles" / "pmc_traffic.json"
     if not path.exists():
-        return None
+        return None, None
     try:
-        return json.loads(path.read_text()).get(f"{kernel}@{workload}", {}).get("traffic_bytes")
+        table = json.loads(path.read_text())
+        entry = table.get(f"{kernel}@{workload}", {})
+        source = f"profiles/pmc_traffic.json (library source {table.get('_library_source_sha16', 'unknown')})"
+        return entry.get("traffic_bytes"), source
     except (ValueError, AttributeError):
-        return None
+        return None, None
+
+
+def library_source_sha16():
+    """Hash of the kernel sources the loaded library was built from (csrc/ and include/)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in sorted((ROOT / "mgrrmsnorm_amd" / "csrc").glob("*.h*")) + sorted((ROOT / "include").glob("*.h")):
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def ceiling(wl, launches=200):
+    """What plain streaming kernels reach on this workload's own tensors, in this run."""
+    t_copy = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe("copy", i, st))
+    t_2r1w = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe("2r1w", i, st))
+    n = wl.tensor_bytes
+    return {"tensor_bytes": n, "copy_us": round(t_copy * 1e6, 3), "copy_GB/s": round(2 * n / t_copy / 1e9, 1),
+            "2r1w_us": round(t_2r1w * 1e6, 3), "2r1w_GB/s": round(3 * n / t_2r1w / 1e9, 1)}
+
+
+def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
+    """Forward + backward through the nn.Module (megagemm.RMSNorm), eager, as a user calls it:
+    host-side cost included.  Wall time per call over `iters` calls, inputs rotating; best and
+    median of `repeats` runs (torch's autograd engine hands the backward pass to a worker
+    thread, and that hand-over alone is worth 25-45 us per call, in two distinct regimes).
+    `torch_floor` is the same loop around `(x * 2).backward(dy)`: what torch itself costs."""
+    import megagemm
+    from mgrrmsnorm_amd import ops
+
+    td = TORCH[dtype]
+    e = ESIZE[dtype]
+    norm = megagemm.RMSNorm(cols, 1e-6).cuda().to(td)
+    nsets = max(2, -(-4 * INFINITY_CACHE_BYTES // (4 * rows * cols * e)))
+    g = torch.Generator(device="cuda").manual_seed(7)
+    xs = [torch.randn((rows, cols), generator=g, device="cuda").to(td).requires_grad_(True) for _ in range(nsets)]
+    dys = [torch.randn((rows, cols), generator=g, device="cuda").to(td) for _ in range(nsets)]
+
+    def call(i):
+        x = xs[i % nsets]
+        x.grad = None
+        norm.weight.grad = None
+        norm(x).backward(dys[i % nsets])
+
+    def fwd_only(i):
+        with torch.no_grad():
+            norm(xs[i % nsets])
+
+    def torch_floor(i):
+        x = xs[i % nsets]
+        x.grad = None
+        (x * 2).backward(dys[i % nsets])
+
+    out = {"binding": ops.backend(), "shape": f"{rows}x{cols} {dtype}"}
+    for key, fn, nbytes in (("fwd_bwd", call, 5 * rows * cols * e + 2 * cols * e + 4 * cols),
+                            ("fwd", fwd_only, 2 * rows * cols * e + cols * e), ("torch_floor", torch_floor, 0)):
+        for i in range(20):
+            fn(i)
+        torch.cuda.synchronize()
+        runs = []
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            for i in range(iters):
+                fn(i)
+            torch.cuda.synchronize()
+            runs.append((time.perf_counter() - t0) / iters)
+        runs.sort()
+        out[key + "_us_per_call"] = round(runs[0] * 1e6, 2)
+        out[key + "_us_per_call_median"] = round(runs[len(runs) // 2] * 1e6, 2)
+        if nbytes:
+            out[key + "_GB/s"] = round(nbytes / runs[0] / 1e9, 1)
+    return out
+
+
+# The benchmark configurations other than the headline one, timed with a few launches each
+# (per-kernel microseconds and algorithmic GB/s): fp16 forward at 4096 x 4096, the large bf16
+# shape, the 65536-row hidden-size sweep in both 2-byte types, and the SwiGLU activation.
+CONFIGS = (["rmsnorm_fwd_4096x4096_fp16", "rmsnorm_fwd_bwd_16384x8192_bf16"]
+           + [f"rmsnorm_fwd_bwd_65536x{c}_{d}" for c in (768, 2048, 4100, 5120, 16384) for d in ("bf16", "fp16")]
+           + ["swiglu_fwd_bwd_8192x11008_bf16"])
+
+
+def time_configs(lib):
+    import gc
+
+    out = {}
+    for name in CONFIGS:
+        wl = make_workload(lib, name, nsets=0)
+        big = wl.step_bytes > 1e9
+        rec = {}
+        for kname, nbytes in wl.kernels.items():
+            t = time_kernel(wl, kname, launches=20 if big else 100)
+            short = kname.split("_")[-1]
+            rec[short + "_us"] = round(t * 1e6, 2)
+            rec[short + "_GB/s"] = round(nbytes / t / 1e9)
+        out[name] = rec
+        log(f"[bench] config {name}: {rec}")
+        del wl
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
 
 
 SWEEP = [
@@ -327,12 +459,20 @@ def main():
                     help="input/output buffer sets the steps rotate over; 0 = enough to exceed four times the "
                          "256 MiB Infinity Cache (the reported configuration), 1 = everything stays cache resident")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--option", action="append", default=[], metavar="KEY=VALUE",
+                    help="tuning override passed to mg_set_option before anything is timed (repeatable)")
+    ap.add_argument("--surface", choices=["abi", "module"], default="abi",
+                    help="'module' also times forward+backward through megagemm.RMSNorm (eager, host cost included) "
+                         "at the workload's shape; the default run reports it for the headline shape anyway")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the per-kernel figures of the other benchmark configurations ('configs' in the JSON)")
     ap.add_argument("--sweep", action="store_true",
                     help="additionally time every configuration of the hidden-size sweep, the large RMSNorm shape "
                          "and the SwiGLU shape (per-kernel and per-step GB/s, table on stderr, 'sweep' in the JSON)")
     ap.add_argument("--calibrate-copies", type=int, default=0,
                     help="also launch this many plain copies of one activation tensor (mg_copy_bytes), so that a "
-                         "counter profile of this run holds a kernel of known HBM traffic")
+                         "counter profile of this run holds a kernel of known HBM traffic, and as many streaming "
+                         "probes of each kind (mg_stream_probe) over the workload's tensors")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -344,6 +484,9 @@ def main():
     from mgrrmsnorm_amd import _lib
     lib = _lib.load()
     torch.cuda.set_device(0)
+    for kv in args.option:
+        key, _, val = kv.partition("=")
+        _lib.set_option(key, int(val))
     wl = make_workload(lib, args.workload, args.buffer_sets)
     log(f"[bench] {wl.name}: {wl.step_bytes / 1e6:.1f} MB algorithmic per step, {wl.nsets} buffer sets, "
         f"device {torch.cuda.get_device_name(0)}")
@@ -356,6 +499,8 @@ def main():
             s_ = wl.sets[i % wl.nsets]
             rc = lib.mg_copy_bytes(s_[dst_key].data_ptr(), s_[src_key].data_ptr(), nbytes, stream_ptr())
             assert rc == 0, lib.mg_last_error()
+            wl.probe("copy", i, stream_ptr())      # the streaming yardsticks, so a profile holds them too
+            wl.probe("2r1w", i, stream_ptr())
         torch.cuda.synchronize()
         log(f"[bench] calibration: {args.calibrate_copies} copies of {nbytes} bytes (traffic 2 x {nbytes} each)")
 
@@ -380,11 +525,18 @@ def main():
         t = time_kernel(wl, name)
         kern[name] = {"us": round(t * 1e6, 3), "GB/s": round(nbytes / t / 1e9, 1), "bytes": nbytes}
         log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch, {nbytes / t / 1e9:.0f} GB/s")
+    for name in getattr(wl, "extra_kernels", []):
+        t = time_kernel(wl, name)
+        kern[name] = {"us": round(t * 1e6, 3)}
+        log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch")
     dom = wl.dominant
     achieved = kern[dom]["GB/s"]
+    traffic, traffic_source = committed_traffic(dom, wl.name)
     roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": committed_traffic(dom, wl.name),
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "algorithmic_bytes": kern[dom]["bytes"], "avg_launch_us": kern[dom]["us"]}
+    ceil = ceiling(wl)
+    log(f"[bench] ceiling on the same tensors: {ceil}")
 
     out = {
         "metric": "RMSNorm fwd+bwd HBM GB/s at [4096x4096] bf16" if wl.name == "rmsnorm_fwd_bwd_4096x4096_bf16"
@@ -394,14 +546,23 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
         "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
-        "kernels": kern, "roofline": roofline,
+        "kernels": kern, "roofline": roofline, "ceiling": ceil, "library_source_sha16": library_source_sha16(),
     }
-    if args.sweep:
-        del wl
-        out["sweep"] = sweep(lib)
+    if isinstance(wl, RmsNormWorkload) and (args.surface == "module" or not args.no_configs):
+        out["module"] = time_module_surface(wl.rows, wl.cols, wl.dtype)
+        log(f"[bench] nn.Module surface: {out['module']}")
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(make_workload(lib, args.workload) if args.sweep else wl)
+        out["cpu_baseline"] = cpu_baseline(wl)
         log(f"[bench] cpu baseline: {out['cpu_baseline']}")
+    del wl
+    import gc
+
+    gc.collect()
+    torch.cuda.empty_cache()
+    if not args.no_configs:
+        out["configs"] = time_configs(lib)
+    if args.sweep:
+        out["sweep"] = sweep(lib)
     print(json.dumps(out), flush=True)
 
 

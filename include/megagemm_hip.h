@@ -20,9 +20,12 @@
  *     launched and mg_last_error() returns a thread-local, human-readable message;
  *   - arguments are validated before any HIP call, so argument errors are reported on a
  *     machine without a GPU too;
- *   - rows == 0 (or M == 0) is valid and launches nothing;
- *   - re-entrant and callable from any thread (the autograd engine calls backward from
- *     its own device thread).
+ *   - rows == 0 (or M == 0) is valid and launches no work on x (backward still zeroes dW);
+ *   - callable from any thread (the autograd engine calls backward from its own device
+ *     thread) and re-entrant: the functions declared here keep no state of their own
+ *     between calls except the partials array of mg_rmsnorm_bwd_noalloc, documented
+ *     there.  The launch shapes they choose can be overridden for the
+ *     whole process through megagemm_hip_tuning.h; nothing else is process-wide.
  */
 #ifndef MEGAGEMM_HIP_H
 #define MEGAGEMM_HIP_H
@@ -153,42 +156,6 @@ int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void
  */
 int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t H, int dtype,
                   void* stream);
-
-/*
- * Reports the launch shape mg_rmsnorm_fwd (backward == 0) or mg_rmsnorm_bwd (backward != 0)
- * takes for rows of `cols` elements; no counterpart in
- * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
- * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
- * workgroup per row, *vectors_per_thread = 0).  *generic = 0 with *vectors_per_thread = 0
- * means a row too wide for registers, streamed twice by a 1024-thread workgroup.
- * *threads_per_row below 64 means that
- * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
- * 640 bytes when the pitch is not a multiple of 16 bytes).
- */
-int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
-                           int* vectors_per_thread, int* workgroup_threads);
-
-/*
- * Measurement aid with no counterpart in the reference: a plain device-to-device copy of
- * `bytes` (a multiple of 16; both pointers 16-byte aligned) done by one kernel that moves
- * one 16-byte vector per thread.  Its HBM traffic is exactly 2*bytes, which makes it the
- * yardstick for calibrating hardware traffic counters when profiling the other kernels.
- */
-int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
-
-/*
- * Tuning hook (not needed for normal use): overrides one launch parameter for the
- * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
- * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
- * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
- * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
- * the current one; -1 = automatic), "swiglu_unroll",
- * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
- * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
- * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for
- * an unknown key.  Values that do not fit a given problem are ignored for that call.
- */
-int mg_set_option(const char* key, int value);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,68 @@
+/*
+ * megagemm_hip_tuning.h -- measurement and tuning aids of libmegagemm_hip.so.
+ *
+ * Nothing here has a counterpart in the reference, and no normal caller needs it: the
+ * operators are declared in megagemm_hip.h.  These functions exist for benchmarks, profiler
+ * runs and tests.  mg_set_option changes PROCESS-WIDE state: it is not synchronised with
+ * calls running on other threads (a call reads each option once when it starts), and while
+ * an override is in force the launch shape, the workspace shape that
+ * mg_rmsnorm_bwd_workspace reports and hence the summation order of dW depend on it.
+ */
+#ifndef MEGAGEMM_HIP_TUNING_H
+#define MEGAGEMM_HIP_TUNING_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Reports the launch shape mg_rmsnorm_fwd (backward == 0) or mg_rmsnorm_bwd (backward != 0)
+ * takes for rows of `cols` elements; no counterpart in
+ * the reference (whose launchers always use 256 threads per row, src/rmsnorm_kernel.cu:530).
+ * Host-only: needs no device.  *generic = 1 means the element-wise kernels (one 256-thread
+ * workgroup per row, *vectors_per_thread = 0).  *generic = 0 with *vectors_per_thread = 0
+ * means a row too wide for registers, streamed twice by a 1024-thread workgroup.
+ * *threads_per_row below 64 means that
+ * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
+ * 640 bytes when the pitch is not a multiple of 16 bytes).
+ */
+int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
+                           int* vectors_per_thread, int* workgroup_threads);
+
+/*
+ * Measurement aid with no counterpart in the reference: a plain device-to-device copy of
+ * `bytes` (a multiple of 16; both pointers 16-byte aligned) done by one kernel that moves
+ * one 16-byte vector per thread.  Its HBM traffic is exactly 2*bytes, which makes it the
+ * yardstick for calibrating hardware traffic counters when profiling the other kernels.
+ */
+int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
+
+/*
+ * Streaming yardstick: one kernel that moves `bytes` (a multiple of 16; 16-byte aligned
+ * pointers) with the same 16-byte non-temporal buffer accesses as the operators, 4 KiB per
+ * workgroup.  b == NULL: dst = a (one read, one write per byte); otherwise dst = a + b as
+ * 32-bit words (two reads, one write).  The time such a launch takes at a given size is
+ * the ceiling for an operator with the same read/write mix at that size.
+ */
+int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void* stream);
+
+/*
+ * Tuning hook (not needed for normal use): overrides one launch parameter for the
+ * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
+ * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
+ * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
+ * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
+ * the current one; -1 = automatic), "swiglu_unroll",
+ * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
+ * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
+ * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for
+ * an unknown key.  Values that do not fit a given problem are ignored for that call.
+ */
+int mg_set_option(const char* key, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MEGAGEMM_HIP_TUNING_H */

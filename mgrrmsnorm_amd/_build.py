@@ -1,9 +1,10 @@
-"""Build recipe for libmegagemm_hip.so (hipcc, gfx950 only).
+"""Build recipe for libmegagemm_hip.so (hipcc, gfx950 only) and for the torch extension
+over it (`_binding`, host-only C++ compiled with g++).
 
-The library is built in-tree, next to this file, so that a built copy travels with the
-source tree.  `python -m mgrrmsnorm_amd._build` rebuilds it; `build()` is what the
-package's own entry points call.  Replaces the reference's CUDAExtension recipe
-(setup.py:23-41) and its Makefile (Makefile:9-26).
+Both are built in-tree, next to this file, so that built copies travel with the source
+tree.  `python -m mgrrmsnorm_amd._build` rebuilds them; `build()` is what the package's own
+entry points call.  Replaces the reference's CUDAExtension recipe (setup.py:23-41) and its
+Makefile (Makefile:9-26).
 """
 from __future__ import annotations
 
@@ -11,6 +12,7 @@ import os
 import shutil
 import subprocess
 import sys
+import sysconfig
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
@@ -19,6 +21,9 @@ CSRC = PKG_DIR / "csrc"
 INCLUDE = PKG_DIR.parent / "include"
 LIB_PATH = PKG_DIR / "libmegagemm_hip.so"
 OBJ_DIR = PKG_DIR / "csrc" / "_obj"
+
+BINDING_NAME = "_binding"
+BINDING_PATH = PKG_DIR / f"{BINDING_NAME}{sysconfig.get_config_var('EXT_SUFFIX')}"
 
 ARCH = "gfx950"
 
@@ -58,16 +63,54 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write("\n".join(rest) + "\n")
 
 
-def build(jobs: int | None = None, verbose: bool = False) -> Path:
-    """Compile every translation unit for gfx950 and link libmegagemm_hip.so."""
+def build_binding(verbose: bool = False, out_dir: Path | None = None, lib_dir: Path | None = None) -> Path:
+    """Compile csrc/torch_binding.cpp into the extension module `_binding`: plain C++ built
+    with g++ against torch's headers and libraries and linked to libmegagemm_hip.so, which it
+    finds next to itself at run time ($ORIGIN)."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    lib_dir = lib_dir or PKG_DIR
+    target = (out_dir or PKG_DIR) / BINDING_PATH.name
+    if not (lib_dir / LIB_PATH.name).exists():
+        raise RuntimeError(f"build {LIB_PATH.name} first")
+    cxx = os.environ.get("CXX") or shutil.which("g++")
+    if not cxx:
+        raise RuntimeError("no C++ compiler found (looked at $CXX and g++)")
+    torch_libs = ce.library_paths()
+    tmp = target.with_suffix(".so.tmp")
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-DTORCH_EXTENSION_NAME={BINDING_NAME}",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{INCLUDE}", *[f"-I{p}" for p in ce.include_paths()],
+           f"-I{sysconfig.get_paths()['include']}", "-I/opt/rocm/include",
+           str(CSRC / "torch_binding.cpp"), "-o", str(tmp),
+           *[f"-L{p}" for p in torch_libs], "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip",
+           "-ltorch_hip", f"-L{lib_dir}", "-lmegagemm_hip", "-Wl,-rpath,$ORIGIN",
+           *[f"-Wl,-rpath,{p}" for p in torch_libs]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    _run(cmd)
+    os.replace(tmp, target)
+    return target
+
+
+def build(jobs: int | None = None, verbose: bool = False, binding: bool = True, out_dir: Path | None = None) -> Path:
+    """Compile every translation unit for gfx950, link libmegagemm_hip.so, then build the
+    torch extension over it (binding=False skips that: the ctypes binding needs no compiler
+    beyond hipcc).  out_dir: where the two files (and the intermediate objects) go instead of
+    the package directory."""
     hipcc = find_hipcc()
-    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    out_dir = Path(out_dir) if out_dir else None
+    obj_dir = (out_dir / "_obj") if out_dir else OBJ_DIR
+    lib_path = (out_dir / LIB_PATH.name) if out_dir else LIB_PATH
+    obj_dir.mkdir(parents=True, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     objs = []
 
     def compile_one(unit):
         src, stem, defs = unit
-        obj = OBJ_DIR / f"{stem}.o"
+        obj = obj_dir / f"{stem}.o"
         cmd = [hipcc, *COMMON_FLAGS, *defs, "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -76,12 +119,14 @@ def build(jobs: int | None = None, verbose: bool = False) -> Path:
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(compile_one, UNITS))
-    tmp = LIB_PATH.with_suffix(".so.tmp")
+    tmp = lib_path.with_suffix(".so.tmp")
     _run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(tmp)])
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, lib_path)
+    if binding:
+        build_binding(verbose=verbose, out_dir=out_dir, lib_dir=out_dir)
+    return lib_path
 
 
 if __name__ == "__main__":
-    path = build(verbose="-v" in sys.argv)
-    print(f"built {path}")
+    path = build(verbose="-v" in sys.argv, binding="--no-binding" not in sys.argv)
+    print(f"built {path}" + ("" if "--no-binding" in sys.argv else f" and {BINDING_PATH}"))

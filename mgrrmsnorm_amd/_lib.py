@@ -1,8 +1,10 @@
 """ctypes binding of libmegagemm_hip.so (the C ABI declared in include/megagemm_hip.h).
 
-This is the only module that touches the shared library.  It takes the place of the
-reference's pybind11 extension module `rmsnorm_cuda_ops` (pytorch_binding/binding.cpp)
-and of the Triton launch sites in megagemm/swiglu.py:100-107,122-129.
+Together with the compiled extension `_binding` (csrc/torch_binding.cpp, preferred by
+mgrrmsnorm_amd.ops when it is built) this takes the place of the reference's pybind11
+extension module `rmsnorm_cuda_ops` (pytorch_binding/binding.cpp) and of the Triton launch
+sites in megagemm/swiglu.py:100-107,122-129.  The tuning and measurement entry points
+(include/megagemm_hip_tuning.h) are reachable through this module only.
 
 There is no CPU fallback: if the library is missing or a call fails, a RuntimeError is
 raised with the library's own message.
@@ -28,7 +30,7 @@ _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
 
-# name -> (restype, argtypes); mirrors include/megagemm_hip.h one to one
+# name -> (restype, argtypes); mirrors include/megagemm_hip.h and megagemm_hip_tuning.h one to one
 SIGNATURES = {
     "mg_abi_version": (_int, []),
     "mg_last_error": (ctypes.c_char_p, []),
@@ -41,6 +43,7 @@ SIGNATURES = {
     "mg_swiglu_fwd": (_int, [_vp, _vp, _i64, _i64, _int, _vp]),
     "mg_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mg_copy_bytes": (_int, [_vp, _vp, _i64, _vp]),
+    "mg_stream_probe": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "mg_rmsnorm_launch_info": (_int, [_int, _i64, _int] + [ctypes.POINTER(_int)] * 4),
 }
 
@@ -125,6 +128,6 @@ class device_of:
 def set_option(key: str, value: int) -> None:
     """Tuning hook (mg_set_option); also drops the workspace shapes remembered by ops."""
     check(load().mg_set_option(key.encode(), int(value)), "mg_set_option")
-    from . import ops
+    from . import ops_ctypes
 
-    ops._workspace_shapes.clear()
+    ops_ctypes._workspace_shapes.clear()

@@ -65,9 +65,11 @@ def _report(title, rows):
     print("=" * 64)
 
 
-def bench_swiglu(dtype=torch.float16):
+def bench_swiglu(dtype=torch.float16, configs=None, warmup: int = 10, iterations: int = 100):
+    """Block forward, PyTorch baseline against this package with the same weights; returns
+    {(batch, seq, d_model): {"pytorch_ms": (mean, std), "hip_ms": (mean, std), "max_diff": float}}."""
     results = {}
-    for batch, seq, d_model in SWIGLU_CONFIGS:
+    for batch, seq, d_model in (SWIGLU_CONFIGS if configs is None else configs):
         torch.cuda.reset_peak_memory_stats()
         x = torch.randn(batch, seq, d_model, device="cuda", dtype=dtype)
         ours = MegaGemmTriton(d_model).cuda().to(dtype)
@@ -76,8 +78,8 @@ def bench_swiglu(dtype=torch.float16):
             ours.w12.weight[: ours.hidden] = base.w1.weight
             ours.w12.weight[ours.hidden:] = base.w2.weight
             ours.w3.weight.copy_(base.w3.weight)
-            t_base = time_calls(lambda: base(x))
-            t_ours = time_calls(lambda: ours(x))
+            t_base = time_calls(lambda: base(x), warmup, iterations)
+            t_ours = time_calls(lambda: ours(x), warmup, iterations)
             diff = (base(x) - ours(x)).abs().max().item()
         _report(f"SwiGLU block forward  batch={batch} seq={seq} d_model={d_model} hidden={ours.hidden} {dtype}",
                 [("PyTorch native", *t_base), ("mgrrmsnorm_amd (HIP)", *t_ours)])
@@ -90,9 +92,11 @@ def bench_swiglu(dtype=torch.float16):
     return results
 
 
-def bench_rmsnorm(dtype=torch.float16):
+def bench_rmsnorm(dtype=torch.float16, configs=None, warmup: int = 10, iterations: int = 100):
+    """Forward, PyTorch formula and torch.nn.RMSNorm against this package; returns
+    {(batch, seq, hidden): {"formula_ms", "native_ms", "hip_ms": (mean, std), "max_diff": float}}."""
     results = {}
-    for batch, seq, hidden in RMSNORM_CONFIGS:
+    for batch, seq, hidden in (RMSNORM_CONFIGS if configs is None else configs):
         x = torch.randn(batch, seq, hidden, device="cuda", dtype=dtype)
         ours = RMSNorm(hidden, 1e-6).cuda().to(dtype)
         native = torch.nn.RMSNorm(hidden, eps=1e-6).cuda().to(dtype)
@@ -102,9 +106,9 @@ def bench_rmsnorm(dtype=torch.float16):
             return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
 
         with torch.no_grad():
-            t_formula = time_calls(formula)
-            t_native = time_calls(lambda: native(x))
-            t_ours = time_calls(lambda: ours(x))
+            t_formula = time_calls(formula, warmup, iterations)
+            t_native = time_calls(lambda: native(x), warmup, iterations)
+            t_ours = time_calls(lambda: ours(x), warmup, iterations)
             diff = (formula().float() - ours(x).float()).abs().max().item()
         _report(f"RMSNorm forward  batch={batch} seq={seq} hidden={hidden} {dtype}",
                 [("PyTorch formula", *t_formula), ("torch.nn.RMSNorm", *t_native), ("mgrrmsnorm_amd (HIP)", *t_ours)])
@@ -112,7 +116,8 @@ def bench_rmsnorm(dtype=torch.float16):
         print(f"tokens per second: PyTorch formula {tokens / t_formula[0] * 1e3:,.0f}, "
               f"this package {tokens / t_ours[0] * 1e3:,.0f}")
         print(f"max |difference| vs the formula = {diff:.6f}")
-        results[(batch, seq, hidden)] = {"formula_ms": t_formula, "native_ms": t_native, "hip_ms": t_ours}
+        results[(batch, seq, hidden)] = {"formula_ms": t_formula, "native_ms": t_native, "hip_ms": t_ours,
+                                         "max_diff": diff}
     return results
 
 

@@ -18,7 +18,7 @@
 // workgroup per row, with the same 16-byte accesses.
 //
 // Generic family: one 256-thread workgroup per row, element-wise loads, two passes over
-// the row; used on request, and for rows beyond registers that end in half a dword.
+// the row; nothing selects it by itself, it runs on request only (the force_generic option).
 #pragma once
 #include "mg_device.hpp"
 

@@ -12,8 +12,7 @@ namespace {
 // Zero-fill of the partial matrix for rows == 0 (a kernel rather than a memset node, so
 // that the call behaves the same under stream capture).
 __global__ void __launch_bounds__(256) fill_zero_f32(float* __restrict__ p, long n) {
-    const long i = (long)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0.0f;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) p[i] = 0.0f;
 }
 
 // Plain 16-byte copy, one vector per thread: the yardstick the HBM traffic counters are
@@ -21,6 +20,27 @@ __global__ void __launch_bounds__(256) fill_zero_f32(float* __restrict__ p, long
 __global__ void __launch_bounds__(256) copy_vec16(u32x4* __restrict__ dst, const u32x4* __restrict__ src, long n) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) dst[i] = src[i];
+}
+
+// Streaming yardsticks with the accesses the operators use (16-byte buffer loads/stores with
+// the non-temporal bit, 4 KiB per workgroup): a copy (b == nullptr) or dst = a + b word by
+// word (two reads, one write).  What these reach at a given size bounds any kernel with the
+// same read/write mix.
+template <bool TWO_READS>
+__global__ void __launch_bounds__(256) stream_probe(char* __restrict__ dst, const char* __restrict__ a,
+                                                    const char* __restrict__ b, long bytes, int xcd_group) {
+    const long chunk = 256L * 16;
+    const long c = xcd_remap(blockIdx.x, gridDim.x, xcd_group);
+    const long left = bytes - c * chunk;
+    const u32 n = left >= chunk ? (u32)chunk : (u32)left;
+    const u32 off = threadIdx.x * 16u;
+    Words<4> v = buf_load<4, kStream>(make_rsrc(a + c * chunk, n), off);
+    if constexpr (TWO_READS) {
+        const Words<4> w = buf_load<4, kStream>(make_rsrc(b + c * chunk, n), off);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v.v[j] += w.v[j];
+    }
+    buf_store<4, kStream>(make_rsrc(dst + c * chunk, n), off, v);
 }
 
 // units handled by one launch stay below 2^31 so that 32-bit indices cannot wrap
@@ -214,9 +234,20 @@ hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s) {
     return hipGetLastError();
 }
 
+hipError_t launch_stream_probe(void* dst, const void* a, const void* b, long bytes, int xcd_group, hipStream_t s) {
+    const long n = (bytes + 4095) / 4096;
+    if (n <= 0) return hipSuccess;
+    if (b == nullptr)
+        stream_probe<false><<<dim3((unsigned)n), dim3(256), 0, s>>>((char*)dst, (const char*)a, nullptr, bytes, xcd_group);
+    else
+        stream_probe<true><<<dim3((unsigned)n), dim3(256), 0, s>>>((char*)dst, (const char*)a, (const char*)b, bytes, xcd_group);
+    return hipGetLastError();
+}
+
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s) {
     if (n <= 0) return hipSuccess;
-    fill_zero_f32<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>(p, n);
+    const long blocks = (n + 255) / 256;
+    fill_zero_f32<<<dim3((unsigned)(blocks < (1L << 20) ? blocks : (1L << 20))), dim3(256), 0, s>>>(p, n);
     return hipGetLastError();
 }
 

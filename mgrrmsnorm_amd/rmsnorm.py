@@ -4,7 +4,9 @@ Same names, argument order, defaults, parameter name and repr as the reference's
 megagemm/rmsnorm.py:18-78 (`RMSNormFunction.apply(input, weight, epsilon=1e-5)`,
 `RMSNorm(hidden_size, epsilon=1e-5)` with a `weight` parameter of ones), so a state_dict or a
 call site written for the reference works unchanged.  The arithmetic runs in hand-written
-HIP kernels reached through mgrrmsnorm_amd.ops; there is no other code path.
+HIP kernels reached through mgrrmsnorm_amd.ops; there is no other code path.  `RMSNorm` calls
+the operator's C++ autograd node when the compiled extension is present (no Python in
+backward); `RMSNormFunction` is the same flow as a Python autograd.Function.
 """
 from __future__ import annotations
 
@@ -69,17 +71,10 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size))
 
     def forward(self, input: torch.Tensor) -> torch.Tensor:
-        weight = self.weight
-        if torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad):
-            return RMSNormFunction.apply(input, weight, self.epsilon)
-        # nothing to differentiate (inference, torch.no_grad()): same kernel, without the
-        # autograd node and its saved tensors
-        shape = input.shape
-        if len(shape) < 1:
-            raise RuntimeError("RMSNorm needs at least one dimension")
-        x2d = (input if input.is_contiguous() else input.contiguous()).view(-1, shape[-1])
-        w = weight if weight.is_contiguous() else weight.contiguous()
-        return ops.rmsnorm_forward(x2d, w, self.epsilon)[0].view(shape)
+        # one call: the compiled extension holds the autograd node (same flow as
+        # RMSNormFunction, in C++); without it ops.rmsnorm goes through RMSNormFunction.
+        # Nothing to differentiate (inference, torch.no_grad()): same kernel, no node.
+        return ops.rmsnorm(input, self.weight, self.epsilon)
 
     def extra_repr(self) -> str:
         return f"hidden_size={self.hidden_size}, eps={self.epsilon}"

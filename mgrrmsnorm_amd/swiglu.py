@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import torch
 import torch.nn as nn
+from torch.autograd.function import once_differentiable
 
 from . import ops
 
@@ -31,6 +32,7 @@ class MegaGemmFunction(torch.autograd.Function):
         return out.view(*fused.shape[:-1], hidden_dim)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, grad_output: torch.Tensor):
         (fused,) = ctx.saved_tensors
         hidden_dim = ctx.hidden_dim
@@ -61,13 +63,9 @@ class MegaGemmTriton(nn.Module):
         self.w3 = nn.Linear(self.hidden, d_model, bias=False)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        fused = self.w12(x)
-        if torch.is_grad_enabled() and fused.requires_grad:
-            return self.w3(MegaGemmFunction.apply(fused, self.hidden))
-        # nothing to differentiate: same kernel, without the autograd node
-        fused = fused if fused.is_contiguous() else fused.contiguous()
-        act = ops.swiglu_forward(fused.view(-1, 2 * self.hidden), self.hidden)
-        return self.w3(act.view(*fused.shape[:-1], self.hidden))
+        # the activation's autograd node lives in the compiled extension when that is built
+        # (else MegaGemmFunction); with nothing to differentiate it is the bare kernel
+        return self.w3(ops.swiglu(self.w12(x), self.hidden))
 
     def extra_repr(self) -> str:
         return f"d_model={self.w12.in_features}, hidden={self.hidden} (Triton Accelerated)"

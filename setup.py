@@ -1,7 +1,9 @@
 """Packaging for mgrrmsnorm_amd: `pip install -e .` (or `python setup.py build`) compiles
-libmegagemm_hip.so for gfx950 with hipcc and ships it inside the package, next to the
-ctypes loader.  There is no torch C++ extension to build: the binding is the plain C ABI
-in include/megagemm_hip.h.  (Reference: a CUDAExtension built by nvcc, setup.py:23-41.)
+libmegagemm_hip.so for gfx950 with hipcc and the torch extension `_binding` over its C ABI
+(include/megagemm_hip.h) with g++, and ships both inside the package, next to the ctypes
+loader that serves when no C++ compiler is at hand.  `python setup.py build_hip
+[--out-dir DIR]` runs just that compile step.  (Reference: a CUDAExtension built by nvcc,
+setup.py:23-41.)
 """
 import sys
 from pathlib import Path
@@ -14,25 +16,26 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 
-def _compile_library():
+def _compile_library(out_dir=None):
     from mgrrmsnorm_amd import _build
 
-    print(f"building {_build.LIB_PATH} for {_build.ARCH}")
-    _build.build()
+    print(f"building {_build.LIB_PATH.name} for {_build.ARCH} and {_build.BINDING_PATH.name}"
+          + (f" into {out_dir}" if out_dir else ""))
+    _build.build(out_dir=out_dir)
 
 
 class BuildHip(Command):
-    description = "compile libmegagemm_hip.so with hipcc (gfx950)"
-    user_options = []
+    description = "compile libmegagemm_hip.so with hipcc (gfx950) and the torch extension over it"
+    user_options = [("out-dir=", None, "directory for the built files (default: inside the package)")]
 
     def initialize_options(self):
-        pass
+        self.out_dir = None
 
     def finalize_options(self):
         pass
 
     def run(self):
-        _compile_library()
+        _compile_library(self.out_dir)
 
 
 class BuildPyWithHip(build_py):
@@ -60,7 +63,7 @@ setup(
     extras_require={"dev": ["pytest", "numpy"]},
     packages=["mgrrmsnorm_amd", "megagemm"],
     py_modules=["rmsnorm_cuda_ops"],
-    package_data={"mgrrmsnorm_amd": ["libmegagemm_hip.so", "csrc/*.hip", "csrc/*.hpp", "csrc/tools/*.hip"]},
-    data_files=[("include", ["include/megagemm_hip.h"])],
+    package_data={"mgrrmsnorm_amd": ["libmegagemm_hip.so", "_binding*.so", "csrc/*.hip", "csrc/*.hpp", "csrc/*.cpp"]},
+    data_files=[("include", ["include/megagemm_hip.h", "include/megagemm_hip_tuning.h"])],
     cmdclass={"build_hip": BuildHip, "build_py": BuildPyWithHip, "develop": DevelopWithHip},
 )

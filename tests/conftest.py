@@ -39,3 +39,16 @@ def oracle():
 
     _oracle.build()
     return _oracle
+
+
+def pytest_terminal_summary(terminalreporter):
+    """How many elements the parity tests let through the cancellation floor (oracle/compare.py)."""
+    try:
+        from oracle import compare
+    except ImportError:
+        return
+    lines = compare.stats_lines()
+    if lines:
+        terminalreporter.section("cancellation-floor accounting")
+        for ln in lines:
+            terminalreporter.write_line(ln)

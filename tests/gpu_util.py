@@ -1,19 +1,6 @@
-"""Helpers for the GPU parity tests: seeded inputs, raw C-ABI calls on torch tensors, and
-the comparison rules.
-
-Comparison rules (from the build's stated tolerances):
-  fp32 outputs       |got - ref| <= 1e-5 * |ref|  (+ the cancellation floor below)
-  fp16/bf16 outputs  at most 1 unit in the last place away from the double-precision
-                     oracle rounded once to the output type
-  cancellation floor dx and d_gate are sums of terms of either sign:
-                       dx[r,c] = s*dy*w  -  sum_j x[r,c]*(s^3/C)*dy[r,j]*w[j]*x[r,j]
-                     Where the terms nearly cancel, no fp32 evaluation (the reference's
-                     included) resolves the result to 1 ulp of itself; what fp32 arithmetic
-                     does guarantee is the forward error bound of a computed sum, a few ulps
-                     of the sum of the terms' magnitudes.  An element therefore also passes
-                     when |got - ref| <= 8 * 2^-24 * (sum of |terms|).
-  dW                 on the fp32 buffer, scale-aware: max|got - ref| / max|ref| <= 1e-3 and
-                     ||got - ref||_2 / ||ref||_2 <= 1e-3; bit-identical from run to run.
+"""Helpers for the GPU parity tests: seeded inputs and raw C-ABI calls on torch tensors.
+The comparison rules (1e-5 relative for fp32, 1 ulp for fp16/bf16, the counted cancellation
+floor for dx and d_gate, the scale-aware dW metric) live in oracle/compare.py.
 """
 from __future__ import annotations
 
@@ -23,11 +10,12 @@ import numpy as np
 import torch
 
 import oracle
+from oracle import compare
 from mgrrmsnorm_amd import _lib
 
 DTYPES = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16}
 CODES = {"fp32": 0, "fp16": 1, "bf16": 2}
-FP32_ULP = 2.0 ** -24
+FP32_ULP = compare.FP32_ULP
 
 
 def lib():
@@ -128,46 +116,9 @@ def swiglu_bwd(dh: torch.Tensor, gu: torch.Tensor, H: int, dtype: str):
 
 # -------------------------------------------------------------------------- comparisons
 
-def assert_matches(got: torch.Tensor, ref64: np.ndarray, dtype: str, what: str, floor: np.ndarray | None = None):
-    """Apply the output rule of this module's docstring to one tensor."""
-    ref64 = np.asarray(ref64, dtype=np.float64)
-    g_store = as_np(got, dtype)
-    g64 = oracle.to_f32(g_store, dtype).astype(np.float64)
-    assert g64.shape == ref64.shape, f"{what}: shape {g64.shape} vs {ref64.shape}"
-    assert np.isfinite(g64).all(), f"{what}: non-finite values in the output"
-    err = np.abs(g64 - ref64)
-    if dtype == "fp32":
-        bad = err > 1e-5 * np.abs(ref64) + 1e-37
-        detail = lambda i: f"rel err {err[i] / max(abs(ref64[i]), 1e-300):.3e}"
-    else:
-        ulps = oracle.ulp_distance(g_store, oracle.round_to(ref64, dtype), dtype)
-        bad = ulps > 1
-        detail = lambda i: f"{ulps[i]} ulp"
-    if floor is not None:
-        bad &= err > 8 * FP32_ULP * floor
-    if bad.any():
-        idx = np.unravel_index(np.argmax(np.where(bad, err, -1.0)), err.shape)
-        raise AssertionError(
-            f"{what} [{dtype}]: {int(bad.sum())} of {bad.size} elements out of tolerance; worst at {idx}: "
-            f"got {g64[idx]!r}, ref {ref64[idx]!r}, {detail(idx)}")
-
-
-def assert_dw(dw_f32: torch.Tensor, ref64: np.ndarray, what="dW"):
-    got = dw_f32.detach().cpu().numpy().astype(np.float64)
-    assert np.isfinite(got).all(), f"{what}: non-finite"
-    scale = max(np.abs(ref64).max(), 1e-300)
-    e_max = np.abs(got - ref64).max() / scale
-    e_l2 = np.linalg.norm(got - ref64) / max(np.linalg.norm(ref64), 1e-300)
-    assert e_max <= 1e-3 and e_l2 <= 1e-3, f"{what}: max-scaled err {e_max:.3e}, l2 err {e_l2:.3e}"
-    return e_max, e_l2
-
-
-def dx_floor(x, dy, w, s):
-    """Sum of the magnitudes of the terms dx is made of (see the module docstring)."""
-    x, dy, w, s = (np.asarray(a, dtype=np.float64) for a in (x, dy, w, s))
-    cols = x.shape[1]
-    gwx = np.abs(dy * w * x).sum(-1, keepdims=True)
-    return np.abs(s[:, None] * dy * w) + np.abs(x) * (s[:, None] ** 3 / cols) * gwx
+assert_matches = compare.assert_matches
+assert_dw = compare.assert_dw
+dx_floor = compare.dx_floor
 
 
 def rmsnorm_reference(x_cpu, dy_cpu, w_cpu, eps, dtype):
@@ -190,9 +141,4 @@ def swiglu_reference(gu_cpu, dh_cpu, dtype):
         return h, None, None
     dh32 = oracle.to_f32(as_np(dh_cpu, dtype), dtype)
     d = oracle.swiglu_bwd_f64(dh32, gu32)
-    H = gu32.shape[1] // 2
-    g, u = gu32[:, :H].astype(np.float64), gu32[:, H:].astype(np.float64)
-    sig = 1.0 / (1.0 + np.exp(-g))
-    base = np.abs(dh32.astype(np.float64) * u * sig)
-    floor = np.concatenate([base * (1.0 + np.abs(g) * (1.0 - sig)), np.zeros_like(base)], axis=1)
-    return h, d, floor
+    return h, d, compare.swiglu_floor(dh32, gu32)

@@ -161,6 +161,44 @@ def test_swiglu_block_against_unfused_baseline(dtype, tol):
     assert (block.w12.weight.grad - gw).abs().max().item() < 2e-2 * gw.abs().max().item()
 
 
+def test_swiglu_block_at_the_benchmark_size():
+    """The SwiGLU block configuration of the benchmark at its own size: d_model 4096,
+    hidden 11008 (hidden_multiple = 2.6875), x [8, 1024, 4096] bf16, weights N(0, 0.02), against
+    the unfused PyTorch block with the same weights (benchmark_swiglu.py:40-58,85-89).  The two
+    sides differ by the rounding of bf16 intermediates and by the order in which two matmuls
+    of different shape add up their terms, hence tolerances rather than ulps; the activation
+    itself is held to 1 ulp against the oracle in test_swiglu_gpu.py."""
+    from megagemm import MegaGemmTriton
+
+    torch.manual_seed(42)
+    d_model, dtype = 4096, torch.bfloat16
+    block = MegaGemmTriton(d_model, hidden_multiple=2.6875).cuda().to(dtype)
+    assert block.hidden == 11008 and block.w12.weight.shape == (22016, 4096) and block.w3.weight.shape == (4096, 11008)
+    base = _UnfusedSwiGLU(d_model, block.hidden).cuda().to(dtype)
+    with torch.no_grad():
+        for p in base.parameters():
+            p.normal_(0.0, 0.02)
+        block.w12.weight[: block.hidden] = base.w1.weight
+        block.w12.weight[block.hidden:] = base.w2.weight
+        block.w3.weight.copy_(base.w3.weight)
+    x = torch.randn(8, 1024, d_model, device="cuda", dtype=dtype)
+    xa, xb = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    ya, yb = block(xa), base(xb)
+    assert ya.shape == (8, 1024, d_model)
+    diff = (ya.float() - yb.float())
+    scale = yb.float().abs().max().item()
+    assert diff.abs().max().item() < 2e-2 * scale
+    assert (diff.norm() / yb.float().norm()).item() < 1e-2
+    g = torch.randn_like(ya)
+    ya.backward(g)
+    yb.backward(g)
+    for got, ref in ((xa.grad, xb.grad), (block.w3.weight.grad, base.w3.weight.grad),
+                     (block.w12.weight.grad, torch.cat([base.w1.weight.grad, base.w2.weight.grad]))):
+        err = (got.float() - ref.float())
+        assert err.abs().max().item() < 3e-2 * ref.float().abs().max().item()
+        assert (err.norm() / ref.float().norm()).item() < 1e-2
+
+
 def test_activation_function_gradient_layout():
     """MegaGemmFunction.backward returns [d_gate | d_up] for the fused input and None for
     hidden_dim (megagemm/swiglu.py:131)."""

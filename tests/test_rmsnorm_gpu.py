@@ -242,11 +242,12 @@ def _tiled(block: torch.Tensor, reps: int) -> torch.Tensor:
 
 FULL = [
     ("bf16", 16384, 8192),    # forward+backward configuration
-    ("bf16", 65536, 768),
-    ("fp16", 65536, 2048),
-    ("bf16", 65536, 4100),
-    ("fp16", 65536, 5120),
-    ("bf16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
+    # the hidden-size sweep at its full 65536 rows, both 2-byte types
+    ("bf16", 65536, 768), ("fp16", 65536, 768),
+    ("bf16", 65536, 2048), ("fp16", 65536, 2048),
+    ("bf16", 65536, 4100), ("fp16", 65536, 4100),
+    ("bf16", 65536, 5120), ("fp16", 65536, 5120),
+    ("bf16", 65536, 16384), ("fp16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
     ("fp32", 70000, 16388),   # 4.6 GB per tensor, rows 4-byte aligned only: offsets beyond 2^32
     ("bf16", 2097152, 128),   # rows narrower than a wave: 8 rows per wave, 262144 waves
     ("fp16", 1048576, 256),

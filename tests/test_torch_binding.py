@@ -1,41 +1,43 @@
-"""The compiled torch extension over the C ABI (tests/integration/torch_binding.cpp): the
-binding a maintainer of the reference would swap in for pytorch_binding/binding.cpp.  It is
-built by tests/integration/build_binding.py (or __graft_entry__.build()); these tests skip
-when it has not been built."""
-import importlib
-import sys
-from pathlib import Path
-
+"""The compiled torch extension over the C ABI (mgrrmsnorm_amd/csrc/torch_binding.cpp, built
+by mgrrmsnorm_amd._build into mgrrmsnorm_amd/_binding*.so): what replaces the reference's
+pytorch_binding/binding.cpp.  It must agree bit for bit with the ctypes binding of the same
+library, and its C++ autograd nodes with the Python autograd.Functions."""
 import numpy as np
 import pytest
 import torch
 
-HERE = Path(__file__).resolve().parent
-
 
 @pytest.fixture(scope="module")
 def binding():
-    sys.path.insert(0, str(HERE / "integration"))
     try:
-        return importlib.import_module("mg_torch_binding")
+        from mgrrmsnorm_amd import _binding
     except ImportError as exc:
-        pytest.skip(f"mg_torch_binding is not built ({exc}); run python tests/integration/build_binding.py")
-    finally:
-        sys.path.pop(0)
+        pytest.fail(f"mgrrmsnorm_amd._binding is not built ({exc}); run python -m mgrrmsnorm_amd._build")
+    return _binding
 
 
 def test_module_surface_and_host_side_checks(binding):
     """Function names and the error text for host tensors follow binding.cpp:9-11,136-139."""
-    assert callable(binding.rmsnorm_forward) and callable(binding.rmsnorm_backward)
+    from mgrrmsnorm_amd import _lib, ops
+
+    for name in ("rmsnorm_forward", "rmsnorm_backward", "rmsnorm_backward_f32", "swiglu_forward", "swiglu_backward",
+                 "rmsnorm", "swiglu"):
+        assert callable(getattr(binding, name)), name
+    assert binding.abi_version() == _lib.ABI_VERSION
+    assert ops.backend() == "extension"      # the package uses it as soon as it is built
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         binding.rmsnorm_forward(torch.ones(2, 8), torch.ones(8), 1e-6)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        binding.swiglu_forward(torch.ones(2, 8), 4)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        binding.rmsnorm(torch.ones(2, 8), torch.ones(8), 1e-6)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
 def test_binding_matches_oracle_and_ctypes_path(binding, dtype):
     import gpu_util as U
-    from mgrrmsnorm_amd import ops
+    from mgrrmsnorm_amd import ops_ctypes
 
     rows, cols, eps = 300, 4096, 1e-6
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=5)
@@ -47,10 +49,92 @@ def test_binding_matches_oracle_and_ctypes_path(binding, dtype):
     np.testing.assert_allclose(s.cpu().numpy(), s_ref, rtol=1e-6)
     U.assert_matches(dx, dx_ref, dtype, "dx", floor=floor)
     assert dw.dtype == wd.dtype   # binding.cpp:90
-    # same library underneath: bit-identical to the ctypes path
-    y2, s2 = ops.rmsnorm_forward(xd, wd, eps)
-    dx2, dw2 = ops.rmsnorm_backward(dyd, xd, wd, s2)
+    dx3, dw32, dwc = binding.rmsnorm_backward_f32(dyd, xd, wd, s)
+    U.assert_dw(dw32, dw_ref)
+    assert torch.equal(dx3, dx) and torch.equal(dwc, dw)
+    dx4, none1, none2 = binding.rmsnorm_backward_f32(dyd, xd, wd, s, need_weight_grad=False)
+    assert none1 is None and none2 is None and torch.equal(dx4, dx)
+    # same library underneath: bit-identical to the ctypes binding
+    y2, s2 = ops_ctypes.rmsnorm_forward(xd, wd, eps)
+    dx2, dw2 = ops_ctypes.rmsnorm_backward(dyd, xd, wd, s2)
     assert torch.equal(y, y2) and torch.equal(s, s2) and torch.equal(dx, dx2) and torch.equal(dw, dw2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_swiglu_binding_matches_oracle_and_ctypes_path(binding, dtype):
+    import gpu_util as U
+    from mgrrmsnorm_amd import ops_ctypes
+
+    M, H = 130, 1376
+    gu = U.cpu_randn((M, 2 * H), 3).to(U.DTYPES[dtype])
+    dh = U.cpu_randn((M, H), 4).to(U.DTYPES[dtype])
+    h_ref, d_ref, floor = U.swiglu_reference(gu, dh, dtype)
+    gud, dhd = gu.cuda(), dh.cuda()
+    h = binding.swiglu_forward(gud, H)
+    d = binding.swiglu_backward(dhd, gud, H)
+    U.assert_matches(h, h_ref, dtype, "h")
+    U.assert_matches(d, d_ref, dtype, "dgu", floor=floor)
+    assert torch.equal(h, ops_ctypes.swiglu_forward(gud, H)) and torch.equal(d, ops_ctypes.swiglu_backward(dhd, gud, H))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cpp_autograd_nodes_match_python_functions(binding, dtype):
+    """binding.rmsnorm / binding.swiglu (autograd nodes in C++) against RMSNormFunction /
+    MegaGemmFunction (Python autograd.Functions over the same kernels): identical bits."""
+    from mgrrmsnorm_amd import MegaGemmFunction, RMSNormFunction
+
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn((3, 50, 768), generator=g).to(dtype).cuda()
+    w = (1 + 0.02 * torch.randn(768, generator=g)).to(dtype).cuda()
+    dy = torch.randn((3, 50, 768), generator=g).to(dtype).cuda()
+    outs = []
+    for fn in (lambda a, b: binding.rmsnorm(a, b, 1e-6), lambda a, b: RMSNormFunction.apply(a, b, 1e-6)):
+        xa, wa = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        y = fn(xa, wa)
+        assert y.shape == x.shape and y.requires_grad
+        y.backward(dy)
+        outs.append((y.detach(), xa.grad, wa.grad))
+    for a, b in zip(*outs):
+        assert a.dtype == b.dtype and torch.equal(a, b)
+    # only the input needs a gradient: no dW is produced
+    xa = x.clone().requires_grad_(True)
+    binding.rmsnorm(xa, w, 1e-6).backward(dy)
+    assert torch.equal(xa.grad, outs[0][1]) and w.grad is None
+    # nothing needs a gradient: plain forward, no node
+    assert binding.rmsnorm(x, w, 1e-6).grad_fn is None
+    with torch.no_grad():
+        assert torch.equal(binding.rmsnorm(x.clone().requires_grad_(True), w, 1e-6), outs[0][0])
+
+    H = 344
+    gu = torch.randn((4, 33, 2 * H), generator=g).to(dtype).cuda()
+    dh = torch.randn((4, 33, H), generator=g).to(dtype).cuda()
+    outs = []
+    for fn in (binding.swiglu, MegaGemmFunction.apply):
+        ga = gu.clone().requires_grad_(True)
+        h = fn(ga, H)
+        assert h.shape == (4, 33, H)
+        h.backward(dh)
+        outs.append((h.detach(), ga.grad))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert binding.swiglu(gu, H).grad_fn is None
+    with pytest.raises(RuntimeError, match="2\\*hidden_dim"):
+        binding.swiglu(gu, H + 1)
+
+
+@pytest.mark.gpu
+def test_cpp_autograd_nodes_refuse_a_second_derivative(binding):
+    x = torch.randn((4, 64), device="cuda", requires_grad=True)
+    w = torch.ones(64, device="cuda", requires_grad=True)
+    y = binding.rmsnorm(x, w, 1e-5)
+    (gx,) = torch.autograd.grad(y.sum(), x, create_graph=False)
+    assert not gx.requires_grad
+    y = binding.rmsnorm(x, w, 1e-5)
+    dy = torch.ones_like(y, requires_grad=True)
+    with pytest.raises(RuntimeError, match="differentiate twice"):
+        torch.autograd.grad(y, x, grad_outputs=dy, create_graph=True)
 
 
 @pytest.mark.gpu
@@ -64,3 +148,5 @@ def test_binding_checks_shapes_on_the_gpu(binding):
         binding.rmsnorm_forward(x.double(), torch.ones(64, device="cuda", dtype=torch.float64), 1e-6)
     with pytest.raises(RuntimeError, match="must be contiguous"):
         binding.rmsnorm_forward(x.t(), torch.ones(4, device="cuda", dtype=torch.float16), 1e-6)
+    with pytest.raises(RuntimeError, match="weight dtype"):
+        binding.rmsnorm(x, torch.ones(64, device="cuda", dtype=torch.float32), 1e-6)
