@@ -31,8 +31,10 @@ def test_swiglu_block_benchmark_default_config_list():
     assert benchmarks.RMSNORM_CONFIGS == [(32, 128, 4096)]
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_rmsnorm_benchmark(dtype, capsys):
+# the formula evaluated by torch in the storage type is itself off by up to an ulp of the
+# output (2^-10 relative in fp16, 2^-7 in bf16; |y| reaches about 4 here)
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 1e-2), (torch.bfloat16, 6.5e-2)])
+def test_rmsnorm_benchmark(dtype, tol, capsys):
     from mgrrmsnorm_amd import benchmarks
 
     cfg = (4, 32, 1024)
@@ -40,7 +42,7 @@ def test_rmsnorm_benchmark(dtype, capsys):
     r = res[cfg]
     assert set(r) == {"formula_ms", "native_ms", "hip_ms", "max_diff"}
     assert all(r[k][0] > 0 for k in ("formula_ms", "native_ms", "hip_ms"))
-    assert r["max_diff"] < 1e-2
+    assert r["max_diff"] < tol
     assert "tokens per second" in capsys.readouterr().out
 
 
