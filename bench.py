@@ -7,7 +7,8 @@ A step is one pass of the hot path over one batch of synthetic input that is alr
 resident in HBM.  The default workload is the one the headline metric is quoted on:
 RMSNorm forward + backward (three launches: forward, backward pass 1, dW reduction) at
 [4096 x 4096] bf16.  The last line printed on stdout is one JSON object; `value` is
-algorithmic bytes per step / wall time per step over exactly K steps.
+algorithmic bytes per step / wall time per step over exactly K steps (the median of five
+such readings; all five are in `readings_us_per_step`).
 
 Buffers rotate over several independent sets whose total size exceeds the 256 MB
 Infinity Cache, so consecutive steps do not find their inputs cached.
@@ -197,11 +198,14 @@ def stream_ptr():
     return torch.cuda.current_stream().cuda_stream
 
 
-def time_steps(wl, steps, warmup, launch):
-    """Wall time of exactly `steps` steps, synchronised on both sides. Returns seconds."""
+def time_steps(wl, steps, warmup, launch, repeats=5):
+    """Wall time of exactly `steps` steps, synchronised on both sides, measured `repeats`
+    times (a timed region of 20 steps lasts under a millisecond, so a single reading moves
+    by a few per cent).  Returns the sorted list of the readings in seconds."""
     for i in range(warmup):
         wl.step(i, stream_ptr())
     torch.cuda.synchronize()
+    readings = []
     if launch == "graph":
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
@@ -210,17 +214,21 @@ def time_steps(wl, steps, warmup, launch):
                 wl.step(warmup + i, st)
         graph.replay()            # untimed: first replay uploads the graph
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        return time.perf_counter() - t0
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            readings.append(time.perf_counter() - t0)
+        return sorted(readings)
     st = stream_ptr()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        wl.step(warmup + i, st)
-    torch.cuda.synchronize()
-    return time.perf_counter() - t0
+    for _ in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            wl.step(warmup + i, st)
+        torch.cuda.synchronize()
+        readings.append(time.perf_counter() - t0)
+    return sorted(readings)
 
 
 def time_kernel(wl, name, launches=200, fn=None):
@@ -392,7 +400,7 @@ def sweep(lib):
         if len(cells) == 1:
             cells.append(" " * 22)
         steps = 20 if big else 100
-        ts = time_steps(wl, steps, 5, "eager") / steps
+        ts = time_steps(wl, steps, 5, "eager", repeats=1)[0] / steps
         rec["step"] = {"us": round(ts * 1e6, 2), "GB/s": round(wl.step_bytes / ts / 1e9, 1)}
         cells.append(f"{ts * 1e6:9.1f} us {wl.step_bytes / ts / 1e9:6.0f} GB/s")
         log(f"[sweep] {name:<36} " + " ".join(cells))
@@ -505,10 +513,11 @@ def main():
         log(f"[bench] calibration: {args.calibrate_copies} copies of {nbytes} bytes (traffic 2 x {nbytes} each)")
 
     modes = ["graph", "eager"] if args.launch == "best" else [args.launch]
-    wall = {}
+    wall, readings = {}, {}
     for mode in modes:
         try:
-            wall[mode] = time_steps(wl, args.steps, args.warmup, mode)
+            readings[mode] = time_steps(wl, args.steps, args.warmup, mode)
+            wall[mode] = readings[mode][len(readings[mode]) // 2]      # the median reading
         except RuntimeError as exc:
             if mode == "graph" and len(modes) > 1:      # "best": the eager measurement still stands
                 log(f"[bench] graph launch not measured: {exc}")
@@ -546,6 +555,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
         "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
         "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
+        "readings_us_per_step": {m: [round(t / args.steps * 1e6, 3) for t in r] for m, r in readings.items()},
         "kernels": kern, "roofline": roofline, "ceiling": ceil, "library_source_sha16": library_source_sha16(),
     }
     if isinstance(wl, RmsNormWorkload) and (args.surface == "module" or not args.no_configs):

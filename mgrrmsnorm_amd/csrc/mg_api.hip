@@ -103,6 +103,9 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
         if (need <= kFwdMaxItems && fwd_items_ok(need)) { *cfg = {kVec, tpr, need, 0}; return true; }
     }
     const int target = (items > 0 && items <= kFwdMaxItems) ? items : 2;
+    // 1025-1536 vectors: 512 threads with three vectors each rather than 1024 with two
+    // (10240 bf16 columns: 6.04 against 5.75 TB/s, 12288: 6.03 against 5.87)
+    if (items == 0 && nvec > 1024 && nvec <= 1536) { *cfg = {kVec, 512, 3, 0}; return true; }
     for (int t = 64; t <= 1024; t *= 2) {
         int need = ceil_div(nvec, t);
         if (need == 7) need = 8;

@@ -50,6 +50,8 @@ SHAPES = [
     (31, 8190),
     (65, 5120),
     (33, 16384),
+    (41, 10240),     # 1280 vectors of 2-byte elements: 512 threads with three vectors each
+    (19, 12279),     # the same launch shape, odd width
     (7, 100),
     (5, 33),         # odd width: rows of 2-byte types end in half a dword
     (9, 4099),
