@@ -40,9 +40,10 @@ int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, 
 int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
 
 /*
- * Streaming yardstick: one kernel that moves `bytes` (a multiple of 16; 16-byte aligned
- * pointers) with the same 16-byte non-temporal buffer accesses as the operators, 4 KiB per
- * workgroup.  b == NULL: dst = a (one read, one write per byte); otherwise dst = a + b as
+ * Streaming yardstick: one kernel that moves `bytes` (a multiple of 16; pointers aligned
+ * to 4 bytes at least -- 16 for the aligned case the operators see with row pitches that are
+ * multiples of 16) with the same 16-byte non-temporal buffer accesses as the operators,
+ * 4 KiB per workgroup.  b == NULL: dst = a (one read, one write per byte); otherwise dst = a + b as
  * 32-bit words (two reads, one write).  The time such a launch takes at a given size is
  * the ceiling for an operator with the same read/write mix at that size.
  */

@@ -435,8 +435,8 @@ int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void
         return fail(MG_ERR_INVALID_ARG, "mg_stream_probe: bytes must be a non-negative multiple of 16 below 2^42 (got %lld)",
                     (long long)bytes);
     if (bytes == 0) return MG_OK;
-    if (dst == nullptr || a == nullptr || !aligned(dst, 16) || !aligned(a, 16) || !aligned(b, 16))
-        return fail(MG_ERR_INVALID_ARG, "mg_stream_probe: dst, a (and b, if given) must be 16-byte aligned device pointers");
+    if (dst == nullptr || a == nullptr || !aligned(dst, 4) || !aligned(a, 4) || !aligned(b, 4))
+        return fail(MG_ERR_INVALID_ARG, "mg_stream_probe: dst, a (and b, if given) must be 4-byte aligned device pointers");
     drop_stale_error();
     hipError_t e = launch_stream_probe(dst, a, b, (long)bytes, xcd_group_or(kXcdGroupStreaming), (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_stream_probe: launch", e);
