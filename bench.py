@@ -269,11 +269,11 @@ def committed_traffic(kernel, workload):
 
 
 def library_source_sha16():
-    """Hash of the kernel sources the loaded library was built from (csrc/ and include/)."""
+    """Hash of the kernel and launcher sources the library is built from (csrc/*.hip, *.hpp)."""
     import hashlib
 
     h = hashlib.sha256()
-    for f in sorted((ROOT / "mgrrmsnorm_amd" / "csrc").glob("*.h*")) + sorted((ROOT / "include").glob("*.h")):
+    for f in sorted((ROOT / "mgrrmsnorm_amd" / "csrc").glob("*.h*")):
         h.update(f.name.encode())
         h.update(f.read_bytes())
     return h.hexdigest()[:16]

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define MG_ABI_VERSION 1
+#define MG_ABI_VERSION 2
 
 /* element types; the reference encodes these in function-name suffixes
  * (_fp32/_fp16/_bf16, src/rmsnorm_kernel.h:9-67) */
@@ -99,8 +99,9 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype,
  * w: [cols]; inv_rms: [rows] fp32; dw_partial: [num_partials, ld] fp32 with ld >= cols and
  * ld % 64 == 0 (mg_rmsnorm_bwd_workspace gives suitable values; any num_partials in
  * [1, 65535] is accepted).  Every element of dw_partial[:, 0:cols] is written, in a fixed
- * order that depends only on (rows, cols, dtype, num_partials): results are bit-identical
- * from run to run.  With rows == 0 the workspace is zero-filled.
+ * order that depends only on (rows, cols, dtype, num_partials) -- and on the launch-shape
+ * overrides of megagemm_hip_tuning.h, if a process sets any: results are bit-identical from
+ * run to run.  With rows == 0 the workspace is zero-filled.
  * Limits as for mg_rmsnorm_fwd (the reference caps cols at 16384 / 32768).
  */
 int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, const void* w,

@@ -18,7 +18,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "libmegagemm_hip.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 MG_F32, MG_F16, MG_BF16 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: MG_F32, torch.float16: MG_F16, torch.bfloat16: MG_BF16}

@@ -63,9 +63,11 @@ def test_header_compiles_as_c_and_cxx(tmp_path):
 
 
 def test_abi_version(lib):
-    assert lib.mg_abi_version() == 1
+    from mgrrmsnorm_amd import _lib
+
+    assert lib.mg_abi_version() == _lib.ABI_VERSION == 2
     text = HEADER.read_text()
-    assert re.search(r"#define\s+MG_ABI_VERSION\s+1\b", text)
+    assert re.search(r"#define\s+MG_ABI_VERSION\s+2\b", text)
 
 
 def _err(lib):
