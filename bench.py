@@ -291,9 +291,11 @@ def ceiling(wl, launches=200):
 def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
     """Forward + backward through the nn.Module (megagemm.RMSNorm), eager, as a user calls it:
     host-side cost included.  Wall time per call over `iters` calls, inputs rotating; best and
-    median of `repeats` runs (torch's autograd engine hands the backward pass to a worker
-    thread, and that hand-over alone is worth 25-45 us per call, in two distinct regimes).
-    `torch_floor` is the same loop around `(x * 2).backward(dy)`: what torch itself costs."""
+    median of `repeats` runs.  torch's autograd engine hands the backward pass to a worker
+    thread; when that thread sits on another core the hand-over costs about 20 us more per
+    call than when both share a core, so the loop is also timed with the process pinned to
+    one core (`fwd_bwd_one_core_*`).  `torch_floor` is the same loop around
+    `(x * 2).backward(dy)`: what torch itself costs."""
     import megagemm
     from mgrrmsnorm_amd import ops
 
@@ -320,9 +322,7 @@ def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
         x.grad = None
         (x * 2).backward(dys[i % nsets])
 
-    out = {"binding": ops.backend(), "shape": f"{rows}x{cols} {dtype}"}
-    for key, fn, nbytes in (("fwd_bwd", call, 5 * rows * cols * e + 2 * cols * e + 4 * cols),
-                            ("fwd", fwd_only, 2 * rows * cols * e + cols * e), ("torch_floor", torch_floor, 0)):
+    def timed(fn):
         for i in range(20):
             fn(i)
         torch.cuda.synchronize()
@@ -333,11 +333,39 @@ def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
                 fn(i)
             torch.cuda.synchronize()
             runs.append((time.perf_counter() - t0) / iters)
-        runs.sort()
+        return sorted(runs)
+
+    out = {"binding": ops.backend(), "shape": f"{rows}x{cols} {dtype}"}
+    step_bytes = 5 * rows * cols * e + 2 * cols * e + 4 * cols
+    for key, fn, nbytes in (("fwd_bwd", call, step_bytes), ("fwd", fwd_only, 2 * rows * cols * e + cols * e),
+                            ("torch_floor", torch_floor, 0)):
+        runs = timed(fn)
         out[key + "_us_per_call"] = round(runs[0] * 1e6, 2)
         out[key + "_us_per_call_median"] = round(runs[len(runs) // 2] * 1e6, 2)
         if nbytes:
             out[key + "_GB/s"] = round(nbytes / runs[0] / 1e9, 1)
+    # The same loop with every thread of the process on one core: the calling thread and the
+    # autograd engine's worker then hand over by a context switch instead of waking another
+    # core, which is where the slower of the two regimes comes from.
+    if hasattr(os, "sched_setaffinity"):
+        saved = {}
+        try:
+            one = {sorted(os.sched_getaffinity(0))[0]}
+            for tid in os.listdir("/proc/self/task"):
+                saved[int(tid)] = os.sched_getaffinity(int(tid))
+                os.sched_setaffinity(int(tid), one)
+            runs = timed(call)
+            out["fwd_bwd_one_core_us_per_call"] = round(runs[0] * 1e6, 2)
+            out["fwd_bwd_one_core_us_per_call_median"] = round(runs[len(runs) // 2] * 1e6, 2)
+            out["fwd_bwd_one_core_GB/s"] = round(step_bytes / runs[0] / 1e9, 1)
+        except OSError:
+            pass
+        finally:
+            for tid, mask in saved.items():
+                try:
+                    os.sched_setaffinity(tid, mask)
+                except OSError:
+                    pass
     return out
 
 
