@@ -64,6 +64,24 @@ def _torch_formula(x, w, eps):
     return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
 
 
+def test_cpu_reference_configuration_at_full_size(oracle):
+    """The CPU-runnable benchmark configuration: x [32,128,4096] fp32 ~N(0,1) from seed 42,
+    w = 1 + 0.02 N(0,1), eps = 1e-6, y = x * rsqrt(mean(x^2) + eps) * w.  The literal fp32
+    restatement must agree with the PyTorch formula in fp32 within the reference's own
+    tolerance (max abs < 1e-4, test_rmsnorm.py:79-81) and with its float64 evaluation."""
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn((32, 128, 4096), generator=g, dtype=torch.float32)
+    w = 1 + 0.02 * torch.randn(4096, generator=g, dtype=torch.float32)
+    x2d = x.view(-1, 4096)
+    y32, s32 = oracle.rmsnorm_fwd_f32(x2d.numpy(), w.numpy(), 1e-6)
+    yt = _torch_formula(x, w, 1e-6).view(-1, 4096).numpy()
+    assert y32.shape == (4096, 4096) and s32.shape == (4096,)
+    assert np.abs(y32 - yt).max() < 1e-4
+    y64 = _torch_formula(x2d.double(), w.double(), 1e-6).numpy()
+    np.testing.assert_allclose(y32, y64, rtol=2e-6, atol=1e-7)
+    np.testing.assert_allclose(s32, torch.rsqrt(x2d.double().pow(2).mean(-1) + 1e-6).numpy(), rtol=2e-6)
+
+
 @pytest.mark.parametrize("rows,cols", [(5, 33), (8, 128), (3, 4100)])
 def test_forward_vs_torch_float64(oracle, rows, cols):
     x, w = _rand(rows, cols), _rand(cols)
