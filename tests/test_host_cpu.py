@@ -117,3 +117,29 @@ def test_unsupported_dtype_message():
     with pytest.raises(RuntimeError, match="Unsupported dtype"):
         _lib.dtype_code(torch.float64)
     assert [_lib.dtype_code(d) for d in (torch.float32, torch.float16, torch.bfloat16)] == [0, 1, 2]
+
+
+def test_binding_choice_can_be_forced_to_ctypes():
+    """mgrrmsnorm_amd.ops uses the compiled extension when it is built and the ctypes binding
+    when MGRRMSNORM_BINDING=ctypes is set before the first call; both reject host tensors
+    with the reference's message (binding.cpp:9)."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    code = ("import torch\nfrom mgrrmsnorm_amd import ops\nprint(ops.backend())\n"
+            "try:\n    ops.rmsnorm_forward(torch.ones(2, 8), torch.ones(8), 1e-6)\n"
+            "except RuntimeError as e:\n    print('error:', e)\n")
+    outs = {}
+    for choice in ("", "ctypes"):
+        env = dict(os.environ, MGRRMSNORM_BINDING=choice, PYTHONPATH=str(root))
+        proc = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, stdout=subprocess.PIPE,
+                              stderr=subprocess.STDOUT, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stdout
+        outs[choice] = proc.stdout
+    assert outs["ctypes"].splitlines()[0] == "ctypes"
+    assert outs[""].splitlines()[0] in ("extension", "ctypes")      # extension once it is built
+    for text in outs.values():
+        assert "must be a CUDA tensor" in text

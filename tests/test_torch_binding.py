@@ -150,3 +150,34 @@ def test_binding_checks_shapes_on_the_gpu(binding):
         binding.rmsnorm_forward(x.t(), torch.ones(4, device="cuda", dtype=torch.float16), 1e-6)
     with pytest.raises(RuntimeError, match="weight dtype"):
         binding.rmsnorm(x, torch.ones(64, device="cuda", dtype=torch.float32), 1e-6)
+
+
+@pytest.mark.gpu
+def test_modules_give_the_same_bits_through_either_binding(binding, monkeypatch):
+    """megagemm.RMSNorm / MegaGemmTriton through the compiled extension (C++ autograd nodes)
+    and through the ctypes binding (Python autograd.Functions): same outputs and gradients."""
+    import megagemm
+    from mgrrmsnorm_amd import ops
+
+    torch.manual_seed(3)
+    norm = megagemm.RMSNorm(1024, 1e-6).cuda().to(torch.bfloat16)
+    mlp = megagemm.MegaGemmTriton(1024).cuda().to(torch.bfloat16)
+    x = torch.randn(4, 40, 1024, device="cuda", dtype=torch.bfloat16)
+    g = torch.randn(4, 40, 1024, device="cuda", dtype=torch.bfloat16)
+
+    def run():
+        for p in list(norm.parameters()) + list(mlp.parameters()):
+            p.grad = None
+        xa = x.clone().requires_grad_(True)
+        y = mlp(norm(xa))
+        y.backward(g)
+        return [y.detach(), xa.grad, norm.weight.grad, mlp.w12.weight.grad, mlp.w3.weight.grad]
+
+    assert ops.backend() == "extension"
+    via_extension = run()
+    monkeypatch.setattr(ops, "_binding", None)
+    monkeypatch.setattr(ops, "_resolved", True)
+    assert ops.backend() == "ctypes"
+    via_ctypes = run()
+    for a, b in zip(via_extension, via_ctypes):
+        assert torch.equal(a, b)
