@@ -130,7 +130,8 @@ def rmsnorm_reference(x_cpu, dy_cpu, w_cpu, eps, dtype):
         return y, s, None, None, None
     dy32 = oracle.to_f32(as_np(dy_cpu, dtype), dtype)
     dx, dw = oracle.rmsnorm_bwd_f64(dy32, x32, w32, eps)
-    floor = dx_floor(x32, dy32, w32, s)
+    dx32, _ = oracle.rmsnorm_bwd_f32(dy32, x32, w32, s.astype(np.float32))   # the reference's arithmetic
+    floor = compare.Floor(dx_floor(x32, dy32, w32, s), dx32)
     return y, s, dx, dw, floor
 
 
@@ -141,4 +142,4 @@ def swiglu_reference(gu_cpu, dh_cpu, dtype):
         return h, None, None
     dh32 = oracle.to_f32(as_np(dh_cpu, dtype), dtype)
     d = oracle.swiglu_bwd_f64(dh32, gu32)
-    return h, d, compare.swiglu_floor(dh32, gu32)
+    return h, d, compare.Floor(compare.swiglu_floor(dh32, gu32), oracle.swiglu_bwd_f32(dh32, gu32))
