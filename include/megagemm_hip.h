@@ -128,8 +128,10 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
  * the one mg_rmsnorm_bwd_workspace reports, capped at MG_NOALLOC_SCRATCH_BYTES / (4 * ld);
  * results are bit-identical to the two-call sequence with that number of partial rows.
  * cols above MG_NOALLOC_MAX_COLS is rejected with MG_ERR_UNSUPPORTED.
- * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two
- * streams, two threads) race on it; calls ordered by a stream or by events do not.
+ * All calls on one GPU share that GPU's array, which keeps the last call's contents: nothing
+ * in it has to start at zero, because every partial sum a call reads was written by that same
+ * call first.  Calls that overlap in time on one GPU (two streams, two threads) race on it;
+ * calls ordered by a stream or by events do not.
  */
 #define MG_NOALLOC_SCRATCH_BYTES (16 << 20)
 #define MG_NOALLOC_MAX_COLS 65536
