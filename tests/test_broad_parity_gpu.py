@@ -2,7 +2,12 @@
 the oracle: widths of every class the launch rules distinguish (a few elements, per-head
 widths, ragged and odd widths, thousands of columns up to 17000), base pointers 0-8 elements
 off the allocation's alignment, and every output surrounded by canary elements so that a
-store outside the tensor shows.  Each case is printed before it runs."""
+store outside the tensor shows.  Each case is printed before it runs.
+
+MG_PARITY_CASES (cases per type and operator, default 120) and MG_PARITY_SEED (added to the
+seeds, default 0) widen or move the sweep for a one-off longer run."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -13,7 +18,8 @@ pytestmark = pytest.mark.gpu
 
 EPS = 1e-6
 PAD = 64
-CASES_PER_DTYPE = 120
+CASES_PER_DTYPE = int(os.environ.get("MG_PARITY_CASES", "120"))
+SEED_SHIFT = int(os.environ.get("MG_PARITY_SEED", "0"))
 
 
 def _padded(shape, td, off, src=None):
@@ -32,7 +38,7 @@ def _canaries_intact(buf, off, n):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
 def test_rmsnorm_many_shapes(dtype):
-    rng = np.random.default_rng({"bf16": 101, "fp16": 202, "fp32": 303}[dtype])
+    rng = np.random.default_rng({"bf16": 101, "fp16": 202, "fp32": 303}[dtype] + SEED_SHIFT)
     td = U.DTYPES[dtype]
     L = U.lib()
     for i in range(CASES_PER_DTYPE):
@@ -78,7 +84,7 @@ def test_rmsnorm_many_shapes(dtype):
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
 def test_swiglu_many_shapes(dtype):
-    rng = np.random.default_rng({"bf16": 404, "fp16": 505, "fp32": 606}[dtype])
+    rng = np.random.default_rng({"bf16": 404, "fp16": 505, "fp32": 606}[dtype] + SEED_SHIFT)
     td = U.DTYPES[dtype]
     L = U.lib()
     for i in range(CASES_PER_DTYPE):
