@@ -294,8 +294,11 @@ def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
     median of `repeats` runs.  torch's autograd engine hands the backward pass to a worker
     thread; when that thread sits on another core the hand-over costs about 20 us more per
     call than when both share a core, so the loop is also timed with the process pinned to
-    one core (`fwd_bwd_one_core_*`).  `torch_floor` is the same loop around
-    `(x * 2).backward(dy)`: what torch itself costs."""
+    one core (`fwd_bwd_one_core_*`), and with
+    `torch.autograd.set_multithreading_enabled(False)`, which makes the engine run the backward
+    pass on the calling thread (`fwd_bwd_caller_thread_*`): no hand-over at all, no pinning
+    needed.  `torch_floor` is the same loop around `(x * 2).backward(dy)`: what torch itself
+    costs."""
     import megagemm
     from mgrrmsnorm_amd import ops
 
@@ -344,6 +347,12 @@ def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
         out[key + "_us_per_call_median"] = round(runs[len(runs) // 2] * 1e6, 2)
         if nbytes:
             out[key + "_GB/s"] = round(nbytes / runs[0] / 1e9, 1)
+    if hasattr(torch.autograd, "set_multithreading_enabled"):
+        with torch.autograd.set_multithreading_enabled(False):
+            runs = timed(call)
+        out["fwd_bwd_caller_thread_us_per_call"] = round(runs[0] * 1e6, 2)
+        out["fwd_bwd_caller_thread_us_per_call_median"] = round(runs[len(runs) // 2] * 1e6, 2)
+        out["fwd_bwd_caller_thread_GB/s"] = round(step_bytes / runs[0] / 1e9, 1)
     # The same loop with every thread of the process on one core: the calling thread and the
     # autograd engine's worker then hand over by a context switch instead of waking another
     # core, which is where the slower of the two regimes comes from.
