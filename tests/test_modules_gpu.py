@@ -365,3 +365,27 @@ def test_frozen_weight_skips_the_dw_reduction():
     x.grad = None
     norm(x).sum().backward()
     assert norm.weight.grad is None and torch.equal(x.grad, want)
+
+
+def test_backward_on_the_calling_thread_gives_the_same_bits():
+    """torch.autograd.set_multithreading_enabled(False) makes the engine run the backward pass
+    on the calling thread instead of its device worker; the nodes must not care."""
+    from mgrrmsnorm_amd import MegaGemmTriton, RMSNorm
+
+    torch.manual_seed(11)
+    norm = RMSNorm(2048, 1e-6).cuda().to(torch.bfloat16)
+    mlp = MegaGemmTriton(2048).cuda().to(torch.bfloat16)
+    x = torch.randn(5, 33, 2048, device="cuda", dtype=torch.bfloat16)
+    dy = torch.randn_like(x)
+
+    def grads():
+        xg = x.clone().requires_grad_(True)
+        for p in list(norm.parameters()) + list(mlp.parameters()):
+            p.grad = None
+        mlp(norm(xg)).backward(dy)
+        return [xg.grad.clone()] + [p.grad.clone() for p in list(norm.parameters()) + list(mlp.parameters())]
+
+    want = grads()
+    with torch.autograd.set_multithreading_enabled(False):
+        got = grads()
+    assert all(torch.equal(a, b) for a, b in zip(want, got))
