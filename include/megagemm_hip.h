@@ -132,6 +132,9 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
  * in it has to start at zero, because every partial sum a call reads was written by that same
  * call first.  Calls that overlap in time on one GPU (two streams, two threads) race on it;
  * calls ordered by a stream or by events do not.
+ * The first call on a GPU looks the array's address up (hipGetSymbolAddress: no allocation,
+ * but it may make the runtime load the library's code object); make one call per GPU before
+ * the first stream capture rather than inside it.
  */
 #define MG_NOALLOC_SCRATCH_BYTES (16 << 20)
 #define MG_NOALLOC_MAX_COLS 65536

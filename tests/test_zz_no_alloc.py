@@ -87,3 +87,38 @@ def test_noalloc_zero_rows_gives_zero_dw():
     U.check(U.lib().mg_rmsnorm_bwd_noalloc(None, dw.data_ptr(), None, None, None, w.data_ptr(), None, 0, cols, 0,
                                            U.stream()), "mg_rmsnorm_bwd_noalloc rows=0")
     assert (dw == 0).all()
+
+
+def test_noalloc_under_graph_capture():
+    """What the entry point is for: captured in a HIP graph (after one eager call, which looks
+    the array's address up), every replay reproduces the eager result, with eager work, another
+    shape's call on the shared array and synchronisation between the replays."""
+    rows, cols, dtype = 777, 4096, "bf16"
+    x, dy, w = (t.cuda() for t in U.rmsnorm_inputs(rows, cols, dtype, seed=21))
+    _, s = U.rmsnorm_fwd(x, w, 1e-6, dtype)
+    dx = torch.empty_like(x)
+    dw = torch.empty(cols, dtype=torch.float32, device="cuda")
+    dwc = torch.empty_like(w)
+    L = U.lib()
+
+    def enqueue():
+        U.check(L.mg_rmsnorm_bwd_noalloc(dx.data_ptr(), dw.data_ptr(), dwc.data_ptr(), dy.data_ptr(), x.data_ptr(),
+                                         w.data_ptr(), s.data_ptr(), rows, cols, U.CODES[dtype], U.stream()),
+                "mg_rmsnorm_bwd_noalloc")
+
+    enqueue()
+    torch.cuda.synchronize()
+    want = (dx.clone(), dw.clone(), dwc.clone())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        enqueue()
+    x2, dy2, w2 = (t.cuda() for t in U.rmsnorm_inputs(50, 9000, "fp32", seed=22))
+    _, s2 = U.rmsnorm_fwd(x2, w2, 1e-6, "fp32")
+    for i in range(4):
+        _noalloc(dy2, x2, w2, s2, "fp32")     # overwrites the shared array between replays
+        for t in (dx, dw, dwc):
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(_same_bits(a, b) for a, b in zip((dx, dw, dwc), want)), f"replay {i}"
