@@ -27,6 +27,9 @@ extern "C" {
  * *threads_per_row below 64 means that
  * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
  * 640 bytes when the pitch is not a multiple of 16 bytes).
+ * *vectors_per_thread = -G (G = 1, 2 or 4) means the row-group layout of rows of at most 64
+ * vectors: a lane holds one vector of its row, *threads_per_row (8, 16, 32 or 64) lanes serve
+ * a row, and a wave keeps G groups of 64 / *threads_per_row consecutive rows in flight.
  */
 int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,
                            int* vectors_per_thread, int* workgroup_threads);
@@ -55,7 +58,9 @@ int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void
  * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
  * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
- * the current one; -1 = automatic), "swiglu_unroll",
+ * the current one; -1 = automatic), "narrow_groups" (the row-group layout for rows of at most
+ * 64 vectors: 1, 2 or 4 groups in flight, 0 = never, -1 = automatic; a "fwd_tpr" / "fwd_items" /
+ * "bwd_tpr" / "bwd_block" override switches the automatic choice off), "swiglu_unroll",
  * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
  * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
  * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for

@@ -12,9 +12,43 @@ struct RowCfg {
     int tpr;    // threads per row: 64, 128, 256, 512, 1024; 8, 16 or 32 = several rows per wave
     int items;  // vectors per thread
     int block;  // backward only: threads per workgroup, 1024 or 512
-    int family; // kFamilyResident (rows held in registers) or kFamilyStreaming (rows read twice)
+    int family; // kFamilyResident (rows held in registers), kFamilyStreaming (rows read twice) or
+                // kFamilyGroups (narrow rows, one vector per lane; `items` = row groups in flight)
 };
 constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
+// Rows of at most 64 vectors can also go one vector per lane, `items` groups of 64/tpr rows
+// per wave in flight ("row groups"); `tpr` is then 8, 16, 32 or 64 and at least the row's vectors.
+constexpr int kFamilyGroups = 2;
+constexpr bool groups_ok(long row_bytes, int tpr, int groups) {
+    return (tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64) && (row_bytes + 15) / 16 <= tpr &&
+           (groups == 1 || groups == 2 || groups == 4);
+}
+constexpr int groups_tpr(long row_bytes) {   // 0 = the row has more than 64 vectors
+    const long nvec = (row_bytes + 15) / 16;
+    return nvec <= 8 ? 8 : (nvec <= 16 ? 16 : (nvec <= 32 ? 32 : (nvec <= 64 ? 64 : 0)));
+}
+// Which rows take the row-group layout by default, and with how many groups in flight
+// (0 = the several-vectors-per-lane layout).  From sweeps over 4...512 columns of all three
+// types at 2^18...2^20 rows on MI355X:
+//  - pitch a multiple of 16 bytes: the row-group layout whenever the pitch is not a multiple of
+//    128 bytes (there the other layout writes cache lines in pieces: 80 bf16 columns forward
+//    3.9 -> 5.8 TB/s, backward 4.8 -> 5.7; 200 columns 3.7 -> 5.8 and 5.3 -> 6.0), and for rows
+//    of up to 16 vectors in any case (128 columns: 6.0 -> 6.2 and 6.0 -> 6.1); four groups
+//    forward, two backward (which also keeps the next block's two in flight);
+//  - other pitches: only while a row fills three quarters of its lanes or has at most 8
+//    vectors, and up to 32 vectors (100 bf16 columns: 4.6 -> 5.1 and 4.6 -> 5.1; 129 columns,
+//    17 of 32 lanes: backward 4.2 -> 3.0, so not there).
+constexpr int groups_default(long row_bytes, bool backward) {
+    const long nvec = (row_bytes + 15) / 16;
+    const int tpr = groups_tpr(row_bytes);
+    if (tpr == 0) return 0;
+    if (row_bytes % 16 == 0) {
+        if (row_bytes % 128 == 0 && nvec > 16) return 0;
+        return backward ? 2 : 4;
+    }
+    if (tpr > 32 || !(nvec <= 8 || 4 * nvec >= 3 * tpr)) return 0;
+    return backward ? (nvec <= 16 ? 4 : 2) : 2;
+}
 // Rows that do not fit registers stream through 1024-thread workgroups.
 
 constexpr int kVec = 16;
@@ -54,7 +88,9 @@ constexpr int narrow_default_tpr(long row_bytes, bool backward) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     if (row_bytes % kVec != 0) return nvec <= 24 ? 8 : (nvec <= 32 ? 32 : (nvec <= 40 ? 16 : 0));
     if (backward) return nvec <= 16 ? 8 : (nvec <= 32 ? 16 : (nvec <= 56 ? 32 : 0));
-    return nvec <= 32 ? 8 : (nvec <= 64 ? 16 : (nvec <= 128 ? 32 : 0));
+    // 65-128 vectors: only pitches that are multiples of 128 bytes (others measure 6-11 %
+    // faster with a wave per row and two vectors per lane: 1000 bf16 columns 5.1 -> 5.7 TB/s)
+    return nvec <= 32 ? 8 : (nvec <= 64 ? 16 : (nvec <= 128 && row_bytes % 128 == 0 ? 32 : 0));
 }
 
 struct FwdArgs {

@@ -53,6 +53,34 @@ hipError_t run_narrow(const FwdArgs& a, hipStream_t s) {
     return hipGetLastError();
 }
 
+template <int TPR, int G, bool RAGGED, int POL>
+hipError_t run_groups(const FwdArgs& a, hipStream_t s) {
+    constexpr int RPB = 4 * G * (kWave / TPR);
+    const long grid = (a.rows + RPB - 1) / RPB;
+    rmsnorm_fwd_groups<elem_t, TPR, G, RAGGED, POL><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
+        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+        1.0f / (float)a.cols, a.xcd_group);
+    return hipGetLastError();
+}
+
+// ragged rows (pitch not a multiple of 16 bytes) take the default cache policy, as in the
+// several-vectors-per-lane kernels; the others stream
+template <int TPR, int G>
+hipError_t groups_by_pitch(const FwdArgs& a, hipStream_t s) {
+    const bool ragged = ((long)a.cols * (long)sizeof(elem_t)) % kVec != 0;
+    return ragged ? run_groups<TPR, G, true, kKeep>(a, s) : run_groups<TPR, G, false, kStream>(a, s);
+}
+
+template <int TPR>
+hipError_t groups_by_g(int g, const FwdArgs& a, hipStream_t s) {
+    switch (g) {
+        case 1: return groups_by_pitch<TPR, 1>(a, s);
+        case 2: return groups_by_pitch<TPR, 2>(a, s);
+        case 4: return groups_by_pitch<TPR, 4>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 template <int TPR>
 hipError_t narrow_by_items(int items, const FwdArgs& a, hipStream_t s) {
     if (narrow_items((long)a.cols * (long)sizeof(elem_t), TPR) != items) return hipErrorInvalidValue;
@@ -96,6 +124,15 @@ hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const Fwd
             (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
             1.0f / (float)a.cols);
         return hipGetLastError();
+    }
+    if (cfg.family == kFamilyGroups) {
+        if (!groups_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items)) return hipErrorInvalidValue;
+        switch (cfg.tpr) {
+            case 8: return groups_by_g<8>(cfg.items, a, s);
+            case 16: return groups_by_g<16>(cfg.items, a, s);
+            case 32: return groups_by_g<32>(cfg.items, a, s);
+            default: return groups_by_g<64>(cfg.items, a, s);
+        }
     }
     if (cfg.vec == kVec) return by_tpr<kVec>(cfg.tpr, cfg.items, a, s);
     return hipErrorInvalidValue;

@@ -198,6 +198,244 @@ rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __re
     }
 }
 
+// Narrow rows, one vector per lane ("row groups"): TPR = 8, 16, 32 or 64 lanes per row with
+// TPR >= the row's vectors, and G groups of 64/TPR consecutive rows per wave in flight.
+// Every load or store instruction of a wave then covers one contiguous piece of memory (the
+// idle lanes of a row map to nothing), whatever the row pitch -- the layout for pitches that
+// are not multiples of 128 bytes, where the several-vectors-per-lane layout above writes
+// cache lines in pieces.  Ragged rows as above; POL = cache policy of the activations.
+template <int TPR>
+__device__ __forceinline__ float lanes_sum(float v) {
+    if constexpr (TPR == kWave) return wave_sum(v);
+    else return group_sum<TPR>(v);
+}
+
+template <typename T, int TPR, int G, bool RAGGED, int POL>
+__global__ void __launch_bounds__(256)
+rmsnorm_fwd_groups(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                   const T* __restrict__ w, long rows, int cols, float eps, float inv_cols, int xcd_group) {
+    constexpr int RPG = kWave / TPR;   // rows per group
+    constexpr int RPW = G * RPG;       // rows per wave
+    constexpr int RPB = 4 * RPW;       // rows per workgroup
+    constexpr int EPV = 16 / (int)sizeof(T);
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int lane = tid & (kWave - 1);
+    const int sub = lane / TPR;
+    const int lir = lane % TPR;
+    const long row0 = xcd_remap(blockIdx.x, gridDim.x, xcd_group) * RPB + (long)wave * RPW;
+    const long left = rows - row0;
+    const u32 live_rows = left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = (row_bytes + 15u) / 16u;
+    const long base = live_rows ? row0 * (long)cols : 0;
+    const rsrc_t rx = make_rsrc(x + base, live_rows * row_bytes);
+    const rsrc_t ry = make_rsrc(y + base, live_rows * row_bytes);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+    const bool mine = (u32)lir < nvec;
+    const u32 pos = (u32)lir * 16u;             // where this lane's vector starts in its row
+    const u32 rem = row_bytes - pos;            // what the row holds from there (wraps when !mine)
+    const u32 tail_off = row_bytes - 2u;
+    bool owns_tail = false;
+    if constexpr (RAGGED && sizeof(T) == 2) owns_tail = (row_bytes & 2u) != 0 && (u32)lir == (row_bytes - 1u) / 16u;
+    u32 off[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) off[g] = mine ? (u32)(g * RPG + sub) * row_bytes + pos : kOutOfRange;
+
+    Words<4> xv[G];
+    u32 x_tail[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) xv[g] = buf_load<4, POL>(rx, off[g]);
+    Words<4> wv = buf_load<4, kKeep>(rw, mine ? pos : kOutOfRange);
+    if constexpr (RAGGED) {
+        u32 w_tail = 0;
+#pragma unroll
+        for (int g = 0; g < G; ++g) x_tail[g] = 0;
+        if (owns_tail) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) x_tail[g] = load_b16<POL>(rx, (u32)(g * RPG + sub) * row_bytes + tail_off);
+            w_tail = load_b16<kKeep>(rw, tail_off);
+        }
+        trim_row_vector(wv, rem, w_tail);
+    }
+    float wf[EPV];
+    unpack_vec<T, 4>(wv, wf);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        if constexpr (RAGGED) trim_row_vector(xv[g], rem, x_tail[g]);
+        float f[EPV], o[EPV];
+        unpack_vec<T, 4>(xv[g], f);
+        float ss = 0.0f;
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) ss = __builtin_fmaf(f[k], f[k], ss);
+        ss = lanes_sum<TPR>(ss);
+        const float s = fast_rsqrt(ss * inv_cols + eps);
+        const u32 r = (u32)(g * RPG + sub);
+        if (lir == 0 && r < live_rows && inv_rms != nullptr) inv_rms[row0 + r] = s;
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) o[k] = (f[k] * s) * wf[k];
+        if constexpr (RAGGED) store_row_vector<POL>(ry, off[g], rem, pack_vec<T, 4>(o));
+        else buf_store<4, POL>(ry, off[g], pack_vec<T, 4>(o));
+    }
+}
+
+// Backward pass 1 in the same layout: persistent grid of 512-thread workgroups; wave q walks
+// the blocks of G * 64/TPR consecutive rows q, q + Q, q + 2Q ... (Q = all waves), with the
+// next block requested before the current one is reduced.  dW: 4 or 8 sums per lane (all row
+// groups put the same columns on a lane), then across the rows of a wave by lane shuffles,
+// then across the 8 waves in wave order through LDS; one partial row per workgroup.
+template <typename T, int TPR, int G, bool RAGGED, int POL>
+__global__ void __launch_bounds__(512)
+rmsnorm_bwd_groups(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
+                   const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
+                   long rows, int cols, float inv_cols) {
+    constexpr int BLOCK = 512;
+    constexpr int WAVES = BLOCK / kWave;
+    constexpr int RPG = kWave / TPR;
+    constexpr int RPW = G * RPG;
+    constexpr int EPV = 16 / (int)sizeof(T);
+    constexpr int COVER = TPR * EPV;   // columns one row's lanes cover (>= cols)
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int lane = tid & (kWave - 1);
+    const int sub = lane / TPR;
+    const int lir = lane % TPR;
+    const long nwaves = (long)gridDim.x * WAVES;
+    const long q = (long)blockIdx.x * WAVES + wave;
+    const long nblocks = (rows + RPW - 1) / RPW;
+    const long n_it = (nblocks + nwaves - 1) / nwaves;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const u32 nvec = (row_bytes + 15u) / 16u;
+    const bool mine = (u32)lir < nvec;
+    const u32 pos = (u32)lir * 16u;
+    const u32 rem = row_bytes - pos;
+    const u32 tail_off = row_bytes - 2u;
+    bool owns_tail = false;
+    if constexpr (RAGGED && sizeof(T) == 2) owns_tail = (row_bytes & 2u) != 0 && (u32)lir == (row_bytes - 1u) / 16u;
+    u32 off[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) off[g] = mine ? (u32)(g * RPG + sub) * row_bytes + pos : kOutOfRange;
+
+    float acc[EPV];
+#pragma unroll
+    for (int k = 0; k < EPV; ++k) acc[k] = 0.0f;
+
+    float wf[EPV];
+    {
+        const rsrc_t rw = make_rsrc(w, row_bytes);
+        Words<4> wv = buf_load<4, kKeep>(rw, mine ? pos : kOutOfRange);
+        if constexpr (RAGGED) {
+            u32 w_tail = 0;
+            if (owns_tail) w_tail = load_b16<kKeep>(rw, tail_off);
+            trim_row_vector(wv, rem, w_tail);
+        }
+        unpack_vec<T, 4>(wv, wf);
+    }
+
+    auto live_rows_of = [&](long row0) -> u32 {
+        const long left = rows - row0;
+        return left <= 0 ? 0u : (left < RPW ? (u32)left : (u32)RPW);
+    };
+    auto request = [&](long row0, u32 live, Words<4> (&xo)[G], Words<4> (&go)[G], u32 (&xt)[G], u32 (&gt)[G], float (&so)[G]) {
+        const long base = live ? row0 * (long)cols : 0;
+        const rsrc_t rx = make_rsrc(x + base, live * row_bytes);
+        const rsrc_t rg = make_rsrc(dy + base, live * row_bytes);
+#pragma unroll
+        for (int g = 0; g < G; ++g) xo[g] = buf_load<4, POL>(rx, off[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) go[g] = buf_load<4, POL>(rg, off[g]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            xt[g] = 0; gt[g] = 0; so[g] = 0.0f;
+            if constexpr (RAGGED) {
+                if (owns_tail) {
+                    const u32 at = (u32)(g * RPG + sub) * row_bytes + tail_off;
+                    xt[g] = load_b16<POL>(rx, at);
+                    gt[g] = load_b16<POL>(rg, at);
+                }
+            }
+            const u32 r = (u32)(g * RPG + sub);
+            if (r < live) so[g] = inv_rms[row0 + r];
+        }
+    };
+
+    Words<4> xv[G], gv[G];
+    u32 x_tail[G], g_tail[G];
+    float s[G];
+    long row0 = q * RPW;
+    u32 live = live_rows_of(row0);
+    request(row0, live, xv, gv, x_tail, g_tail, s);
+
+    for (long it = 0; it < n_it; ++it) {
+        const long nrow0 = row0 + nwaves * RPW;
+        const u32 nlive = live_rows_of(nrow0);
+        Words<4> nxv[G], ngv[G];
+        u32 nx_tail[G], ng_tail[G];
+        float ns[G];
+        request(nrow0, nlive, nxv, ngv, nx_tail, ng_tail, ns);
+
+        const long base = live ? row0 * (long)cols : 0;
+        const rsrc_t rd = make_rsrc(dx + base, live * row_bytes);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if constexpr (RAGGED) {
+                trim_row_vector(xv[g], rem, x_tail[g]);
+                trim_row_vector(gv[g], rem, g_tail[g]);
+            }
+            float xf[EPV], gf[EPV], o[EPV];
+            unpack_vec<T, 4>(xv[g], xf);
+            unpack_vec<T, 4>(gv[g], gf);
+            float a = 0.0f;
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                const float t = gf[k] * xf[k];
+                a = __builtin_fmaf(t, wf[k], a);
+                acc[k] = __builtin_fmaf(t, s[g], acc[k]);
+            }
+            a = lanes_sum<TPR>(a);
+            const float c2 = a * (s[g] * s[g]) * s[g] * inv_cols;
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s[g], -(xf[k] * c2));
+            if constexpr (RAGGED) store_row_vector<POL>(rd, off[g], rem, pack_vec<T, 4>(o));
+            else buf_store<4, POL>(rd, off[g], pack_vec<T, 4>(o));
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            xv[g] = nxv[g]; gv[g] = ngv[g];
+            x_tail[g] = nx_tail[g]; g_tail[g] = ng_tail[g];
+            s[g] = ns[g];
+        }
+        row0 = nrow0; live = nlive;
+    }
+
+    // rows of one group: lanes lir, lir + TPR, lir + 2*TPR, ... hold the same columns
+#pragma unroll
+    for (int k = 0; k < EPV; ++k)
+#pragma unroll
+        for (int d = TPR; d < kWave; d *= 2) acc[k] += __shfl_xor(acc[k], d);
+
+    // waves of the workgroup, in wave order
+    __shared__ float dwbuf[COVER];
+    for (int g = 0; g < WAVES; ++g) {
+        if (wave == g && sub == 0) {
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) {
+                if (g == 0) dwbuf[lir * EPV + k] = acc[k];
+                else dwbuf[lir * EPV + k] += acc[k];
+            }
+        }
+        __syncthreads();
+    }
+    float* out = dw_part + (long)blockIdx.x * ld;
+    const int lim = ld < COVER ? ld : COVER;
+    for (int c = tid * 4; c < lim; c += BLOCK * 4) {
+        f32x4 v = {dwbuf[c], dwbuf[c + 1], dwbuf[c + 2], dwbuf[c + 3]};
+        *reinterpret_cast<f32x4*>(out + c) = v;
+    }
+    // columns between COVER and ld (COVER can be as small as 32) belong to no lane
+    for (int c = COVER + tid; c < ld; c += BLOCK) out[c] = 0.0f;
+}
+
 // Backward pass 1 for narrow rows: persistent grid of 512-thread workgroups; each wave walks
 // groups of 64/TPR consecutive rows (group g of wave q: rows (g*Q + q)*RPW ..., Q = all waves),
 // prefetching the next group (ragged rows are trimmed when the data is used, not when it is

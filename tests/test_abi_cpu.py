@@ -160,24 +160,30 @@ def _launch_info(lib, backward, cols, dtype):
     (100000, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # wider than registers hold: 1024 threads stream the row twice
     (100001, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # ... an odd width of a 2-byte type too
     (40000, 2, (0, 1024, 5, 1024), (0, 1024, 0, 1024)),   # the backward pass holds fewer vectors than the forward pass
-    # rows of up to 2 KiB share a wave: 8, 16 or 32 lanes per row;
-    # forward up to 4 vectors per lane (128 vectors), backward up to 2 (56 vectors)
-    (64, 2, (0, 8, 1, 256), (0, 8, 1, 512)),            # 8 vectors: 8 rows per wave
-    (128, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # head dimension 128
+    # rows of up to 1 KiB whose pitch is not a multiple of 128 bytes, and any row of up to 16
+    # vectors: one vector per lane, 8 / 16 / 32 / 64 lanes per row, -G = G row groups in flight
+    (64, 2, (0, 8, -4, 256), (0, 8, -2, 512)),          # 8 vectors: 8 rows per group
+    (128, 2, (0, 16, -4, 256), (0, 16, -2, 512)),       # head dimension 128
+    (80, 2, (0, 16, -4, 256), (0, 16, -2, 512)),        # head dimension 80: 10 of 16 lanes
+    (8, 2, (0, 8, -4, 256), (0, 8, -2, 512)),           # a single vector per row
+    (264, 2, (0, 64, -4, 256), (0, 64, -2, 512)),       # 33 vectors, pitch 528 bytes
+    (100, 2, (0, 16, -2, 256), (0, 16, -4, 512)),       # pitch 200 bytes: the last vector of a row is trimmed
+    (64, 0, (0, 16, -4, 256), (0, 16, -2, 512)),
+    # pitches that are multiples of 128 bytes, 17 vectors and up: several vectors per lane,
+    # 8, 16 or 32 lanes per row; forward up to 4 vectors per lane (128 vectors), backward up to 2 (56)
     (256, 1, (0, 8, 4, 256), (0, 16, 2, 512)),
-    (8, 2, (0, 8, 1, 256), (0, 8, 1, 512)),             # a single vector per row
-    (264, 2, (0, 16, 3, 256), (0, 32, 2, 512)),         # 33 vectors
     (512, 2, (0, 16, 4, 256), (0, 64, 1, 512)),         # 64 vectors: backward takes one wave per row
     (768, 2, (0, 32, 3, 256), (0, 64, 2, 512)),
     (1024, 1, (0, 32, 4, 256), (0, 64, 2, 512)),
     (1032, 2, (0, 64, 3, 256), (0, 128, 2, 512)),        # 129 vectors: one wave per row
-    (100, 2, (0, 8, 2, 256), (0, 8, 2, 512)),           # pitch 200 bytes: the last vector of a row is trimmed
+    (1000, 2, (0, 64, 2, 256), (0, 128, 1, 512)),        # 125 vectors, pitch 2000 bytes: contiguous pieces per instruction
+    # ragged rows that leave too many lanes idle, or are long, keep several vectors per lane
+    (129, 1, (0, 8, 3, 256), (0, 8, 3, 512)),           # 17 vectors would idle 15 of 32 lanes
     (299, 1, (0, 16, 3, 256), (0, 16, 3, 512)),         # 598 bytes, rows only 2-byte aligned
-    (999, 1, (0, 64, 2, 256), (0, 64, 2, 512)),         # 1998 bytes: too long for that to pay
-    (64, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
+    (999, 1, (0, 64, 2, 256), (0, 64, 2, 512)),         # 1998 bytes
     # fp32: 4 elements per vector, any width is 4-byte aligned
     (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
-    (33, 0, (0, 8, 2, 256), (0, 8, 2, 512)),
+    (33, 0, (0, 8, 2, 256), (0, 8, 2, 512)),            # 132 bytes: 9 vectors would idle 7 of 16 lanes
     (16384, 0, (0, 1024, 4, 1024), (0, 512, 8, 512)),
 ])
 def test_launch_shapes(lib, cols, dtype, fwd, bwd):

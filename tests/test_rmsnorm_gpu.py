@@ -251,8 +251,10 @@ FULL = [
     ("bf16", 65536, 5120), ("fp16", 65536, 5120),
     ("bf16", 65536, 16384), ("fp16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
     ("fp32", 70000, 16388),   # 4.6 GB per tensor, rows 4-byte aligned only: offsets beyond 2^32
-    ("bf16", 2097152, 128),   # rows narrower than a wave: 8 rows per wave, 262144 waves
-    ("fp16", 1048576, 256),
+    ("bf16", 2097152, 128),   # rows narrower than a wave, one vector per lane: 16 rows per wave in flight
+    ("bf16", 2097152, 80),    # ... at a pitch of 160 bytes
+    ("fp16", 1342144, 100),   # ... at a pitch of 200 bytes: every row's last vector is trimmed
+    ("fp16", 1048576, 256),   # several vectors per lane: 8 rows per wave
 ]
 
 
@@ -435,6 +437,66 @@ def test_every_narrow_row_shape(dtype, tpr, cols):
     U.assert_matches(dx, dx_ref, dtype, f"dx tpr={tpr}", floor=floor)
     U.assert_dw(dw, dw_ref)
     assert torch.isfinite(part).all(), "padding columns of a partial row were left unwritten"
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("groups", [1, 2, 4])
+@pytest.mark.parametrize("cols", [8, 24, 64, 72, 80, 128, 200, 264, 512, 1, 3, 45, 100, 127, 250, 500])   # from 1 on: ragged pitches
+def test_every_row_group_shape(dtype, groups, cols):
+    """Rows of at most 64 vectors with one vector per lane on 8, 16, 32 or 64 lanes and 1, 2 or
+    4 groups of rows per wave in flight, whatever the automatic choice takes; the row count
+    leaves the last wave a partial block of rows."""
+    import ctypes
+
+    rows = 333
+    esize = 4 if dtype == "fp32" else 2
+    nvec = -(-cols * esize // 16)
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=77 + cols)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    L = U.lib()
+    U.check(L.mg_set_option(b"narrow_groups", groups))
+    try:
+        for backward in (0, 1):
+            out = [ctypes.c_int(0) for _ in range(4)]
+            U.check(L.mg_rmsnorm_launch_info(backward, cols, U.CODES[dtype], *[ctypes.byref(o) for o in out]))
+            if nvec <= 64:
+                assert out[2].value == -groups and out[1].value >= nvec and out[1].value in (8, 16, 32, 64)
+            else:
+                assert out[2].value > 0      # too long for the layout: the request is ignored
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+        dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    finally:
+        U.check(L.mg_set_option(b"narrow_groups", -1))
+    U.assert_matches(y, y_ref, dtype, f"y groups={groups}")
+    np.testing.assert_allclose(s.cpu().numpy(), s_ref, rtol=1e-6)
+    U.assert_matches(dx, dx_ref, dtype, f"dx groups={groups}", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    assert torch.isfinite(part).all(), "padding columns of a partial row were left unwritten"
+
+
+def test_row_groups_can_be_switched_off():
+    """narrow_groups = 0 sends every narrow row to the several-vectors-per-lane kernels."""
+    import ctypes
+
+    L = U.lib()
+    U.check(L.mg_set_option(b"narrow_groups", 0))
+    try:
+        for cols in (64, 80, 100, 264):
+            for backward in (0, 1):
+                out = [ctypes.c_int(0) for _ in range(4)]
+                U.check(L.mg_rmsnorm_launch_info(backward, cols, 2, *[ctypes.byref(o) for o in out]))
+                assert out[2].value > 0 and out[1].value in (8, 16, 32)
+        x, dy, w = U.rmsnorm_inputs(200, 80, "bf16", seed=5)
+        y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "bf16")
+        xd, dyd, wd = _dev(x, dy, w)
+        y, s = U.rmsnorm_fwd(xd, wd, EPS, "bf16")
+        dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, "bf16")
+    finally:
+        U.check(L.mg_set_option(b"narrow_groups", -1))
+    U.assert_matches(y, y_ref, "bf16", "y, groups off")
+    U.assert_matches(dx, dx_ref, "bf16", "dx, groups off", floor=floor)
+    U.assert_dw(dw, dw_ref)
 
 
 @pytest.mark.parametrize("tpr", [64, 128, 256, 512, 1024])
