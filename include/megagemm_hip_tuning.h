@@ -28,7 +28,7 @@ extern "C" {
  * 64 / *threads_per_row consecutive rows share a wave (rows of at most 2 KiB; at most
  * 640 bytes when the pitch is not a multiple of 16 bytes).
  * *vectors_per_thread = -G (G = 1, 2 or 4) means the row-group layout of rows of at most 64
- * vectors: a lane holds one vector of its row, *threads_per_row (8, 16, 32 or 64) lanes serve
+ * vectors: a lane holds one vector of its row, *threads_per_row (1, 2, 4 ... 64) lanes serve
  * a row, and a wave keeps G groups of 64 / *threads_per_row consecutive rows in flight.
  */
 int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, int* threads_per_row,

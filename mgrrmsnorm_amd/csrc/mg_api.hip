@@ -315,10 +315,7 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
         if (cfg.block == 1024) dflt_per_cu = 2;   // both fit a compute unit; 5.9 against 5.5-5.8 TB/s with one
         // one vector per lane leaves half the bytes in flight: a second workgroup makes up for it
         if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
-        if (cfg.family == kFamilyGroups) {   // rows that fill at most half their lanes: a second workgroup
-            rg = (cfg.block / cfg.tpr) * cfg.items;
-            dflt_per_cu = 2 * ((cols * es + 15) / 16) <= cfg.tpr ? 2 : 1;
-        }
+        if (cfg.family == kFamilyGroups) { rg = (cfg.block / cfg.tpr) * cfg.items; dflt_per_cu = 1; }
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;

@@ -263,16 +263,17 @@ __device__ __forceinline__ long xcd_remap(long id, long count, int group) {
     return base + (within & 7) * group + (within >> 3);
 }
 
-// Sum over groups of 8, 16 or 32 adjacent lanes (rows narrower than a wave): every lane ends
-// up with its group's total.  xor-1 and xor-2 inside quads, then mirror inside half rows (8)
-// and inside 16-lane rows; for 32 the two row sums of each half wave are read with
+// Sum over groups of 1, 2, 4, 8, 16 or 32 adjacent lanes (rows narrower than a wave): every
+// lane ends up with its group's total.  xor-1 and xor-2 inside quads, then mirror inside half
+// rows (8) and inside 16-lane rows; for 32 the two row sums of each half wave are read with
 // v_readlane and added.  A fixed order, no LDS.
 template <int GROUP>
 __device__ __forceinline__ float group_sum(float v) {
-    static_assert(GROUP == 8 || GROUP == 16 || GROUP == 32, "sub-wave rows are 8, 16 or 32 lanes wide");
-    v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
-    v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
-    v += dpp_mov<0x141>(v);  // row_half_mirror: lane i <-> 7 - i of each 8
+    static_assert(GROUP == 1 || GROUP == 2 || GROUP == 4 || GROUP == 8 || GROUP == 16 || GROUP == 32,
+                  "sub-wave rows are 1 to 32 lanes wide");
+    if constexpr (GROUP >= 2) v += dpp_mov<0xB1>(v);   // quad_perm [1,0,3,2]
+    if constexpr (GROUP >= 4) v += dpp_mov<0x4E>(v);   // quad_perm [2,3,0,1]
+    if constexpr (GROUP >= 8) v += dpp_mov<0x141>(v);  // row_half_mirror: lane i <-> 7 - i of each 8
     if constexpr (GROUP >= 16) v += dpp_mov<0x140>(v);  // row_mirror: lane i <-> 15 - i of each 16
     if constexpr (GROUP == 32) {
         const float lo = read_lane(v, 0) + read_lane(v, 16);

@@ -17,15 +17,18 @@ struct RowCfg {
 };
 constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
 // Rows of at most 64 vectors can also go one vector per lane, `items` groups of 64/tpr rows
-// per wave in flight ("row groups"); `tpr` is then 8, 16, 32 or 64 and at least the row's vectors.
+// per wave in flight ("row groups"); `tpr` is then a power of two from 1 to 64 and at least the
+// row's vectors (below 8 lanes per row only with 2 or 4 groups).
 constexpr int kFamilyGroups = 2;
 constexpr bool groups_ok(long row_bytes, int tpr, int groups) {
-    return (tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64) && (row_bytes + 15) / 16 <= tpr &&
-           (groups == 1 || groups == 2 || groups == 4);
+    const bool lanes = tpr == 1 || tpr == 2 || tpr == 4 || tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64;
+    return lanes && (row_bytes + 15) / 16 <= tpr && (groups == 2 || groups == 4 || (groups == 1 && tpr >= 8));
 }
 constexpr int groups_tpr(long row_bytes) {   // 0 = the row has more than 64 vectors
     const long nvec = (row_bytes + 15) / 16;
-    return nvec <= 8 ? 8 : (nvec <= 16 ? 16 : (nvec <= 32 ? 32 : (nvec <= 64 ? 64 : 0)));
+    int t = 1;
+    while (t < nvec && t < 128) t *= 2;
+    return t <= 64 ? t : 0;
 }
 // Which rows take the row-group layout by default, and with how many groups in flight
 // (0 = the several-vectors-per-lane layout).  From sweeps over 4...512 columns of all three

@@ -74,7 +74,9 @@ hipError_t groups_by_pitch(const FwdArgs& a, hipStream_t s) {
 template <int TPR>
 hipError_t groups_by_g(int g, const FwdArgs& a, hipStream_t s) {
     switch (g) {
-        case 1: return groups_by_pitch<TPR, 1>(a, s);
+        case 1:
+            if constexpr (TPR >= 8) return groups_by_pitch<TPR, 1>(a, s);
+            else return hipErrorInvalidValue;
         case 2: return groups_by_pitch<TPR, 2>(a, s);
         case 4: return groups_by_pitch<TPR, 4>(a, s);
         default: return hipErrorInvalidValue;
@@ -128,6 +130,9 @@ hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const Fwd
     if (cfg.family == kFamilyGroups) {
         if (!groups_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items)) return hipErrorInvalidValue;
         switch (cfg.tpr) {
+            case 1: return groups_by_g<1>(cfg.items, a, s);
+            case 2: return groups_by_g<2>(cfg.items, a, s);
+            case 4: return groups_by_g<4>(cfg.items, a, s);
             case 8: return groups_by_g<8>(cfg.items, a, s);
             case 16: return groups_by_g<16>(cfg.items, a, s);
             case 32: return groups_by_g<32>(cfg.items, a, s);

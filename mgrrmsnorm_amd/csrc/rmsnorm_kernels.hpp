@@ -198,7 +198,7 @@ rmsnorm_fwd_narrow(T* __restrict__ y, float* __restrict__ inv_rms, const T* __re
     }
 }
 
-// Narrow rows, one vector per lane ("row groups"): TPR = 8, 16, 32 or 64 lanes per row with
+// Narrow rows, one vector per lane ("row groups"): TPR = 1, 2, 4 ... 64 lanes per row with
 // TPR >= the row's vectors, and G groups of 64/TPR consecutive rows per wave in flight.
 // Every load or store instruction of a wave then covers one contiguous piece of memory (the
 // idle lanes of a row map to nothing), whatever the row pitch -- the layout for pitches that

@@ -161,11 +161,12 @@ def _launch_info(lib, backward, cols, dtype):
     (100001, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # ... an odd width of a 2-byte type too
     (40000, 2, (0, 1024, 5, 1024), (0, 1024, 0, 1024)),   # the backward pass holds fewer vectors than the forward pass
     # rows of up to 1 KiB whose pitch is not a multiple of 128 bytes, and any row of up to 16
-    # vectors: one vector per lane, 8 / 16 / 32 / 64 lanes per row, -G = G row groups in flight
+    # vectors: one vector per lane, 1 ... 64 lanes per row, -G = G row groups in flight
     (64, 2, (0, 8, -4, 256), (0, 8, -2, 512)),          # 8 vectors: 8 rows per group
     (128, 2, (0, 16, -4, 256), (0, 16, -2, 512)),       # head dimension 128
     (80, 2, (0, 16, -4, 256), (0, 16, -2, 512)),        # head dimension 80: 10 of 16 lanes
-    (8, 2, (0, 8, -4, 256), (0, 8, -2, 512)),           # a single vector per row
+    (8, 2, (0, 1, -4, 256), (0, 1, -2, 512)),           # a single vector per row: a lane per row
+    (24, 1, (0, 4, -4, 256), (0, 4, -2, 512)),          # 3 vectors on 4 lanes
     (264, 2, (0, 64, -4, 256), (0, 64, -2, 512)),       # 33 vectors, pitch 528 bytes
     (100, 2, (0, 16, -2, 256), (0, 16, -4, 512)),       # pitch 200 bytes: the last vector of a row is trimmed
     (64, 0, (0, 16, -4, 256), (0, 16, -2, 512)),
