@@ -12,7 +12,11 @@
 // elements ends in half a dword, which one lane moves with 2-byte accesses (RowTail).
 //
 // Narrow family: rows of at most 128 vectors put 8, 16 or 32 lanes on a row, so that one
-// wave carries 8, 4 or 2 consecutive rows (see below).
+// wave carries 8, 4 or 2 consecutive rows, with up to 4 vectors per lane (see below).
+//
+// Row-group family: rows of at most 64 vectors put 1 ... 64 lanes on a row with one vector
+// per lane, and a wave keeps several groups of 64/lanes consecutive rows in flight; every
+// load or store instruction then covers one contiguous piece of memory (see below).
 //
 // Streaming family: rows that do not fit registers are read twice by one 1024-thread
 // workgroup per row, with the same 16-byte accesses.
