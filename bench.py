@@ -84,6 +84,7 @@ class RmsNormWorkload:
         self.name = f"rmsnorm_{'fwd_bwd' if backward else 'fwd'}_{rows}x{cols}_{dtype}"
         self.desc = {"rows": rows, "cols": cols, "eps": 1e-6, "launches_per_step": 3 if backward else 1}
         self.tensor_bytes = rows * cols * e
+        self.row_bytes = cols * e
 
     def _chk(self, rc):
         if rc != 0:
@@ -122,8 +123,13 @@ class RmsNormWorkload:
         s = self.sets[i % self.nsets]
         if kind == "copy":      # the forward pass's mix: one read, one write
             rc = self.lib.mg_stream_probe(s["y"].data_ptr(), s["x"].data_ptr(), None, self.tensor_bytes, st)
-        else:                   # the backward pass's mix: two reads, one write
+        elif kind == "2r1w":    # the backward pass's mix: two reads, one write
             rc = self.lib.mg_stream_probe(s["dx"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), self.tensor_bytes, st)
+        elif kind == "rows_copy":   # the same bytes, but a workgroup owns a whole row, one row each (forward)
+            rc = self.lib.mg_row_probe(s["y"].data_ptr(), s["x"].data_ptr(), None, self.rows, self.row_bytes, 0, st)
+        else:                   # ("rows_2r1w", G): whole rows on a persistent grid of G workgroups (backward pass 1)
+            rc = self.lib.mg_row_probe(s["dx"].data_ptr(), s["x"].data_ptr(), s["dy"].data_ptr(), self.rows,
+                                       self.row_bytes, kind[1], st)
         self._chk(rc)
 
 
@@ -284,8 +290,28 @@ def ceiling(wl, launches=200):
     t_copy = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe("copy", i, st))
     t_2r1w = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe("2r1w", i, st))
     n = wl.tensor_bytes
-    return {"tensor_bytes": n, "copy_us": round(t_copy * 1e6, 3), "copy_GB/s": round(2 * n / t_copy / 1e9, 1),
-            "2r1w_us": round(t_2r1w * 1e6, 3), "2r1w_GB/s": round(3 * n / t_2r1w / 1e9, 1)}
+    out = {"tensor_bytes": n, "copy_us": round(t_copy * 1e6, 3), "copy_GB/s": round(2 * n / t_copy / 1e9, 1),
+           "2r1w_us": round(t_2r1w * 1e6, 3), "2r1w_GB/s": round(3 * n / t_2r1w / 1e9, 1)}
+    # The same bytes when a workgroup must own whole rows (it cannot store a row before it has
+    # seen all of it): one row per workgroup as in the forward pass, and a persistent grid as in
+    # backward pass 1 (best of 1, 2, 4 and 8 workgroups per compute unit).
+    rb = getattr(wl, "row_bytes", 0)
+    if rb and rb % 16 == 0 and rb <= 65536:
+        t = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe("rows_copy", i, st))
+        out["rows_copy_us"] = round(t * 1e6, 3)
+        out["rows_copy_GB/s"] = round(2 * n / t / 1e9, 1)
+        if getattr(wl, "backward", False):
+            best = None
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            for mult in (1, 2, 4, 8):
+                G = cus * mult
+                t = time_kernel(wl, None, launches, fn=lambda i, st: wl.probe(("rows_2r1w", G), i, st))
+                if best is None or t < best[0]:
+                    best = (t, G)
+            out["rows_2r1w_persistent_us"] = round(best[0] * 1e6, 3)
+            out["rows_2r1w_persistent_GB/s"] = round(3 * n / best[0] / 1e9, 1)
+            out["rows_2r1w_persistent_workgroups"] = best[1]
+    return out
 
 
 def time_module_surface(rows, cols, dtype, iters=300, repeats=6):

@@ -53,6 +53,19 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream);
 int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void* stream);
 
 /*
+ * The same traffic with the operators' division of work: one workgroup (256 threads for rows
+ * of up to 4 KiB, 512 up to 16 KiB, 1024 beyond) owns whole rows of `row_bytes` (a multiple of
+ * 16, at most 65536) and walks the rows g, g + G, g + 2G ... of [rows, row_bytes] matrices,
+ * requesting its next row before it stores the current one: dst = a (b == NULL) or
+ * dst = a + b on 32-bit words.  workgroups = 0 (or >= rows) gives every row a workgroup of
+ * its own, as the forward pass does; a smaller number G is a persistent grid, as backward
+ * pass 1 uses.  It shows what the machine delivers when a workgroup has to take a whole row
+ * at a time: the same as 4 KiB pieces for rows of up to 16 KiB, 5-15 % less at 32 KiB.
+ */
+int mg_row_probe(void* dst, const void* a, const void* b, int64_t rows, int64_t row_bytes,
+                 int64_t workgroups, void* stream);
+
+/*
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
  * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target

@@ -44,6 +44,7 @@ SIGNATURES = {
     "mg_swiglu_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp]),
     "mg_copy_bytes": (_int, [_vp, _vp, _i64, _vp]),
     "mg_stream_probe": (_int, [_vp, _vp, _vp, _i64, _vp]),
+    "mg_row_probe": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mg_rmsnorm_launch_info": (_int, [_int, _i64, _int] + [ctypes.POINTER(_int)] * 4),
 }
 

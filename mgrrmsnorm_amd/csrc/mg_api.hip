@@ -469,6 +469,24 @@ int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void
     return MG_OK;
 }
 
+int mg_row_probe(void* dst, const void* a, const void* b, int64_t rows, int64_t row_bytes, int64_t workgroups,
+                 void* stream) {
+    if (rows < 0 || rows >= (1LL << 31))
+        return fail(MG_ERR_INVALID_ARG, "mg_row_probe: rows must be in [0, 2^31) (got %lld)", (long long)rows);
+    if (row_bytes < 16 || row_bytes % 16 != 0 || row_bytes > 65536)
+        return fail(MG_ERR_INVALID_ARG, "mg_row_probe: row_bytes must be a multiple of 16 from 16 to 65536 (got %lld)",
+                    (long long)row_bytes);
+    if (workgroups < 0 || workgroups >= (1LL << 31))
+        return fail(MG_ERR_INVALID_ARG, "mg_row_probe: workgroups must be in [0, 2^31) (got %lld)", (long long)workgroups);
+    if (rows == 0) return MG_OK;
+    if (dst == nullptr || a == nullptr || !aligned(dst, 4) || !aligned(a, 4) || !aligned(b, 4))
+        return fail(MG_ERR_INVALID_ARG, "mg_row_probe: dst, a (and b, if given) must be 4-byte aligned device pointers");
+    drop_stale_error();
+    hipError_t e = launch_row_probe(dst, a, b, (long)rows, (long)row_bytes, (long)workgroups, (hipStream_t)stream);
+    if (e != hipSuccess) return fail_hip("mg_row_probe: launch", e);
+    return MG_OK;
+}
+
 static int check_swiglu(const char* fn, int64_t M, int64_t H, int dtype) {
     if (esize_of(dtype) == 0)
         return fail(MG_ERR_INVALID_ARG, "%s: unknown dtype %d (use 0=fp32, 1=fp16, 2=bf16)", fn, dtype);

@@ -118,6 +118,8 @@ hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const 
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s);
 hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s);
 hipError_t launch_stream_probe(void* dst, const void* a, const void* b, long bytes, int xcd_group, hipStream_t s);
+hipError_t launch_row_probe(void* dst, const void* a, const void* b, long rows, long row_bytes, long workgroups,
+                            hipStream_t s);
 
 // SwiGLU kernel families: aligned 16-byte vectors (needs H*sizeof(T) % 16 == 0 and 16-byte
 // aligned bases), 16-byte vectors at any alignment with ragged half rows, or one element per

@@ -43,6 +43,48 @@ __global__ void __launch_bounds__(256) stream_probe(char* __restrict__ dst, cons
     buf_store<4, kStream>(make_rsrc(dst + c * chunk, n), off, v);
 }
 
+// The same traffic with the operators' work split: a workgroup of BLOCK threads (256 for rows of
+// up to 4 KiB, 512 up to 16 KiB, 1024 beyond) owns whole rows of `row_bytes` (at most 64 KiB), ITEMS vectors per
+// thread, and walks the rows blockIdx.x,
+// blockIdx.x + gridDim.x, ... with the next row requested before the current one is stored --
+// a grid of `rows` workgroups takes one row each, a smaller grid is persistent like backward
+// pass 1.  What this reaches bounds a kernel that must see a whole row before it can store.
+template <bool TWO_READS, int BLOCK, int ITEMS>
+__global__ void __launch_bounds__(BLOCK) row_probe(char* __restrict__ dst, const char* __restrict__ a,
+                                                    const char* __restrict__ b, long rows, u32 row_bytes) {
+    const u32 tid = threadIdx.x;
+    Words<4> av[ITEMS], bv[ITEMS];
+    auto request = [&](long row, Words<4> (&x)[ITEMS], Words<4> (&y)[ITEMS]) {
+        const bool live = row < rows;
+        const long base = live ? row * (long)row_bytes : 0;
+        const rsrc_t ra = make_rsrc(a + base, live ? row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) x[i] = buf_load<4, kStream>(ra, (tid + i * (u32)BLOCK) * 16u);
+        if constexpr (TWO_READS) {
+            const rsrc_t rb = make_rsrc(b + base, live ? row_bytes : 0u);
+#pragma unroll
+            for (int i = 0; i < ITEMS; ++i) y[i] = buf_load<4, kStream>(rb, (tid + i * (u32)BLOCK) * 16u);
+        }
+    };
+    long row = blockIdx.x;
+    request(row, av, bv);
+    for (; row < rows; row += gridDim.x) {
+        Words<4> na[ITEMS], nb[ITEMS];
+        request(row + gridDim.x, na, nb);
+        const rsrc_t rd = make_rsrc(dst + row * (long)row_bytes, row_bytes);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            if constexpr (TWO_READS) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) av[i].v[j] += bv[i].v[j];
+            }
+            buf_store<4, kStream>(rd, (tid + i * (u32)BLOCK) * 16u, av[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) { av[i] = na[i]; if constexpr (TWO_READS) bv[i] = nb[i]; }
+    }
+}
+
 // units handled by one launch stay below 2^31 so that 32-bit indices cannot wrap
 constexpr long kMaxUnitsPerLaunchDefault = 1L << 31;
 std::atomic<long> g_max_units{kMaxUnitsPerLaunchDefault};
@@ -242,6 +284,28 @@ hipError_t launch_stream_probe(void* dst, const void* a, const void* b, long byt
     else
         stream_probe<true><<<dim3((unsigned)n), dim3(256), 0, s>>>((char*)dst, (const char*)a, (const char*)b, bytes, xcd_group);
     return hipGetLastError();
+}
+
+template <bool TWO_READS>
+hipError_t row_probe_by_shape(unsigned grid, void* dst, const void* a, const void* b, long rows, u32 row_bytes,
+                              hipStream_t s) {
+#define MG_ROW_PROBE(B, I) row_probe<TWO_READS, B, I><<<dim3(grid), dim3(B), 0, s>>>((char*)dst, (const char*)a, (const char*)b, rows, row_bytes)
+    const u32 nvec = row_bytes / 16u;
+    if (nvec <= 256) MG_ROW_PROBE(256, 1);
+    else if (nvec <= 512) MG_ROW_PROBE(512, 1);
+    else if (nvec <= 1024) MG_ROW_PROBE(512, 2);
+    else if (nvec <= 2048) MG_ROW_PROBE(1024, 2);
+    else MG_ROW_PROBE(1024, 4);
+#undef MG_ROW_PROBE
+    return hipGetLastError();
+}
+
+hipError_t launch_row_probe(void* dst, const void* a, const void* b, long rows, long row_bytes, long workgroups,
+                            hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    const unsigned grid = (unsigned)(workgroups > 0 && workgroups < rows ? workgroups : rows);
+    return b == nullptr ? row_probe_by_shape<false>(grid, dst, a, b, rows, (u32)row_bytes, s)
+                        : row_probe_by_shape<true>(grid, dst, a, b, rows, (u32)row_bytes, s);
 }
 
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s) {

@@ -41,7 +41,7 @@ def test_header_declares_the_expected_entry_points():
         "mg_rmsnorm_dw_reduce", "mg_rmsnorm_bwd_noalloc", "mg_swiglu_fwd", "mg_swiglu_bwd"])
     # measurement and tuning aids live in a header of their own
     assert _declared_in(TUNING_HEADER) == sorted([
-        "mg_set_option", "mg_copy_bytes", "mg_stream_probe", "mg_rmsnorm_launch_info"])
+        "mg_set_option", "mg_copy_bytes", "mg_stream_probe", "mg_row_probe", "mg_rmsnorm_launch_info"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -140,6 +140,11 @@ def test_copy_bytes_rejects_bad_arguments(lib):
     assert lib.mg_copy_bytes(FAKE, FAKE + 4, 32, None) == -1 and "aligned" in _err(lib)
     assert lib.mg_copy_bytes(None, FAKE, 32, None) == -1
     assert lib.mg_copy_bytes(None, None, 0, None) == 0
+    assert lib.mg_row_probe(FAKE, FAKE, None, 4, 24, 0, None) == -1 and "multiple of 16" in _err(lib)
+    assert lib.mg_row_probe(FAKE, FAKE, None, 4, 65552, 0, None) == -1
+    assert lib.mg_row_probe(FAKE, FAKE, None, -1, 64, 0, None) == -1 and "rows" in _err(lib)
+    assert lib.mg_row_probe(None, FAKE, None, 4, 64, 0, None) == -1
+    assert lib.mg_row_probe(None, None, None, 0, 64, 0, None) == 0
 
 
 def _launch_info(lib, backward, cols, dtype):
