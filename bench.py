@@ -405,7 +405,8 @@ def time_module_surface(rows, cols, dtype, iters=300, repeats=6):
 
 
 # The benchmark configurations other than the headline one, timed with a few launches each
-# (per-kernel microseconds and algorithmic GB/s): fp16 forward at 4096 x 4096, the large bf16
+# (per-kernel microseconds and algorithmic GB/s, and what the plain streaming probe reaches on
+# the same tensors): fp16 forward at 4096 x 4096, the large bf16
 # shape, the 65536-row hidden-size sweep in both 2-byte types, and the SwiGLU activation.
 CONFIGS = (["rmsnorm_fwd_4096x4096_fp16", "rmsnorm_fwd_bwd_16384x8192_bf16"]
            + [f"rmsnorm_fwd_bwd_65536x{c}_{d}" for c in (768, 2048, 4100, 5120, 16384) for d in ("bf16", "fp16")]
@@ -425,6 +426,11 @@ def time_configs(lib):
             short = kname.split("_")[-1]
             rec[short + "_us"] = round(t * 1e6, 2)
             rec[short + "_GB/s"] = round(nbytes / t / 1e9)
+        # the plain streaming probe on the same tensors: one read + one write, two reads + one write
+        kinds = ["copy"] + (["2r1w"] if getattr(wl, "backward", True) else [])
+        for kind in kinds:
+            t = time_kernel(wl, None, launches=20 if big else 100, fn=lambda i, st: wl.probe(kind, i, st))
+            rec["probe_" + kind + "_GB/s"] = round((2 if kind == "copy" else 3) * wl.tensor_bytes / t / 1e9)
         out[name] = rec
         log(f"[bench] config {name}: {rec}")
         del wl
