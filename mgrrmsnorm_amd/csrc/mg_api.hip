@@ -30,7 +30,7 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1};
 
 // Consecutive logical workgroups one die handles at a time in the one-shot streaming
 // kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
@@ -152,6 +152,19 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         for (int b : {block, 512, 1024})
             if (bwd_cfg_ok(esize, tpr, need, b)) { *cfg = {kVec, tpr, need, b}; return true; }
     }
+    // 2-byte rows of 1537-4096 vectors: 1024 threads with the dW sums in LDS ("bwd_lds" = 0: in
+    // registers; 1 = from 1025 vectors on).  Beyond 2048 vectors the register kernel needs 5-8
+    // vectors per thread at 512 threads and spills (20480 bf16 columns: 4.8 -> 5.9 TB/s,
+    // 32768: 1.2 -> 5.8); at 1537-2048 vectors two such workgroups share a compute unit and
+    // gain 1-5 % (16384 x 16384: 5.77 -> 6.02 TB/s; 65536 x 16384: 5.83 -> 5.87); below that
+    // the register kernel is as fast or faster (10240 columns: 6.0 against 5.8).
+    if (tpr == 0 && block == 0 && opt_bwd_lds.load() != 0) {
+        const int need = ceil_div(nvec, 1024);
+        if (bwd_lds_ok(esize, nvec, need) && (nvec > 1536 || opt_bwd_lds.load() == 1)) {
+            *cfg = {kVec, 1024, need, 1024, kFamilyLdsSums};
+            return true;
+        }
+    }
     // 88-128 vectors at a pitch that is a multiple of 16 but not of 128 bytes: two waves per row with one
     // vector per lane, so that every instruction covers contiguous memory, rather than one
     // wave with two (1000 bf16 columns: 6.0 against 5.4 TB/s; 904: 5.9 against 5.3; below 88
@@ -235,7 +248,7 @@ const char* mg_last_error(void) { return g_err; }
 int mg_set_option(const char* key, int value) {
     if (key == nullptr) return fail(MG_ERR_INVALID_ARG, "mg_set_option: key is NULL");
     struct { const char* k; std::atomic<int>* v; } table[] = {
-        {"narrow_groups", &opt_groups}, {"fwd_tpr", &opt_fwd_tpr},       {"fwd_items", &opt_fwd_items},
+        {"narrow_groups", &opt_groups}, {"bwd_lds", &opt_bwd_lds}, {"fwd_tpr", &opt_fwd_tpr},       {"fwd_items", &opt_fwd_items},
         {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
@@ -316,6 +329,7 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
         // one vector per lane leaves half the bytes in flight: a second workgroup makes up for it
         if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
         if (cfg.family == kFamilyGroups) { rg = (cfg.block / cfg.tpr) * cfg.items; dflt_per_cu = 1; }
+        if (cfg.family == kFamilyLdsSums) dflt_per_cu = cfg.items == 2 ? 2 : 1;   // 64, 96 or 128 KiB of LDS each
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;

@@ -32,6 +32,24 @@ hipError_t run(const BwdArgs& a, hipStream_t s) {
     }
 }
 
+// dW sums in LDS: more dynamic LDS than the 64 KiB a kernel gets without asking
+template <int ITEMS>
+hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
+    if constexpr (sizeof(elem_t) == 2) {
+        constexpr int kLdsBytes = ITEMS * 1024 * (kVec / (int)sizeof(elem_t)) * 4;
+        auto kernel = rmsnorm_bwd_rows_lds<elem_t, ITEMS>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kLdsBytes);
+        if (e != hipSuccess) return e;
+        kernel<<<dim3((unsigned)a.num_partials), dim3(1024), kLdsBytes, s>>>(
+            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+            a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);
+        return hipGetLastError();
+    } else {
+        return hipErrorInvalidValue;
+    }
+}
+
 template <int TPR, int BLOCK>
 hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
     switch (items) {
@@ -136,6 +154,11 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
         return hipGetLastError();
     }
     if (cfg.vec != kVec) return hipErrorInvalidValue;
+    if (cfg.family == kFamilyLdsSums) {
+        const long nvec = ((long)a.cols * (long)sizeof(elem_t) + kVec - 1) / kVec;
+        if (!bwd_lds_ok((int)sizeof(elem_t), nvec, cfg.items)) return hipErrorInvalidValue;
+        return cfg.items == 2 ? run_lds_sums<2>(a, s) : (cfg.items == 3 ? run_lds_sums<3>(a, s) : run_lds_sums<4>(a, s));
+    }
     if (cfg.family == kFamilyGroups) {
         if (!groups_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items)) return hipErrorInvalidValue;
         switch (cfg.tpr) {

@@ -797,6 +797,108 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
 }
 
 // =================================================================================
+// Backward pass 1 for 2-byte rows of 1537-4096 vectors (12 296 ... 32 768 columns): the same
+// persistent scheme with one row slot per 1024-thread workgroup, but the dW sums -- 8 floats
+// per vector, which registers no longer hold next to the row itself once a thread has more
+// than two vectors (with 5-8 vectors per thread at 512 threads the register kernel spills:
+// 4.8 TB/s at 20 480 columns, 1.2 at 32 768) -- live in LDS.  Each thread owns fixed 16-byte
+// slices of it, so no synchronisation is needed.
+//   block = TPR = 1024 threads; grid = P workgroups, one per compute unit (two with 2 vectors);
+//   dynamic LDS = ITEMS * 1024 * (16 / sizeof(T)) floats (64, 96 or 128 KiB)
+// =================================================================================
+template <typename T, int ITEMS>
+__global__ void __launch_bounds__(1024)
+rmsnorm_bwd_rows_lds(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
+                     const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
+                     long rows, int cols, float inv_cols, int xcd_group) {
+    constexpr int TPR = 1024;
+    constexpr int WPR = TPR / kWave;
+    constexpr int EPV = 16 / (int)sizeof(T);
+    constexpr int QPV = EPV / 4;              // 16-byte slices of fp32 sums per vector of T
+    static_assert(ITEMS * TPR * EPV * 4 <= 160 * 1024 - 1024, "the dW sums of a workgroup must fit the LDS of a compute unit");
+
+    const int tid = threadIdx.x;
+    const long nslots = gridDim.x;
+    const long wg = xcd_remap(blockIdx.x, gridDim.x, xcd_group);
+    const long n_it = (rows + nslots - 1) / nslots;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+
+    __shared__ float red[2][WPR];
+    // slice (i, h) of thread t: columns (t + i*TPR)*EPV + 4h .. +3, at sums[(i*QPV + h)*TPR + t];
+    // consecutive threads are 16 bytes apart, so the accesses are free of bank conflicts
+    extern __shared__ f32x4 sums[];
+#pragma unroll
+    for (int j = 0; j < ITEMS * QPV; ++j) sums[j * TPR + tid] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const RowTail tail = row_tail<T, TPR>(cols, row_bytes);
+    Words<4> wv[ITEMS];
+    load_row<4, ITEMS, TPR, kKeep>(wv, make_rsrc(w, row_bytes), tid, tail);
+
+    for (long it = 0; it < n_it; ++it) {
+        const long row = wg + it * nslots;
+        const bool live = row < rows;
+        const long base = live ? row * (long)cols : 0;
+        Words<4> xv[ITEMS], gv[ITEMS];
+        load_row<4, ITEMS, TPR, kStream>(xv, make_rsrc(x + base, live ? row_bytes : 0u), tid, tail);
+        load_row<4, ITEMS, TPR, kStream>(gv, make_rsrc(dy + base, live ? row_bytes : 0u), tid, tail);
+        const float s = live ? inv_rms[row] : 0.0f;
+
+        float a = 0.0f;
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            float xf[EPV], gf[EPV], wf[EPV];
+            unpack_vec<T, 4>(xv[i], xf);
+            unpack_vec<T, 4>(gv[i], gf);
+            unpack_vec<T, 4>(wv[i], wf);
+#pragma unroll
+            for (int h = 0; h < QPV; ++h) {
+                f32x4 acc = sums[(i * QPV + h) * TPR + tid];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float t = gf[4 * h + k] * xf[4 * h + k];
+                    a = __builtin_fmaf(t, wf[4 * h + k], a);
+                    acc[k] = __builtin_fmaf(t, s, acc[k]);
+                }
+                sums[(i * QPV + h) * TPR + tid] = acc;
+            }
+        }
+        a = wave_sum(a);
+        {
+            const int wir = __builtin_amdgcn_readfirstlane(tid / kWave);
+            const int buf = (int)(it & 1);
+            if ((tid & (kWave - 1)) == 0) red[buf][wir] = a;
+            __syncthreads();
+            float t = 0.0f;
+#pragma unroll
+            for (int k = 0; k < WPR; ++k) t += red[buf][k];
+            a = t;
+        }
+        const float c2 = a * (s * s) * s * inv_cols;
+        const rsrc_t rd = make_rsrc(dx + base, live ? row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i) {
+            float xf[EPV], gf[EPV], wf[EPV], o[EPV];
+            unpack_vec<T, 4>(xv[i], xf);
+            unpack_vec<T, 4>(gv[i], gf);
+            unpack_vec<T, 4>(wv[i], wf);
+#pragma unroll
+            for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[k], s, -(xf[k] * c2));
+            store_item<4, TPR, kStream>(rd, tid, i, pack_vec<T, 4>(o), tail);
+        }
+    }
+
+    // every thread writes its own slices of this workgroup's partial row
+    float* out = dw_part + wg * ld;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+        for (int h = 0; h < QPV; ++h) {
+            const int c0 = (tid + i * TPR) * EPV + 4 * h;     // ld % 4 == 0
+            if (c0 < ld) *reinterpret_cast<f32x4*>(out + c0) = sums[(i * QPV + h) * TPR + tid];
+        }
+}
+
+// =================================================================================
 // Backward, generic (any cols / alignment): dx per row, then dW partials per column.
 // =================================================================================
 template <typename T>

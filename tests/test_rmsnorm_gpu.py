@@ -499,6 +499,33 @@ def test_row_groups_can_be_switched_off():
     U.assert_dw(dw, dw_ref)
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("rows,cols", [(33, 12296), (600, 16384), (21, 16383), (33, 16392), (300, 20480), (41, 24576),
+                                       (19, 32768), (7, 32767), (5, 28001)])
+def test_backward_with_the_dw_sums_in_lds(dtype, rows, cols):
+    """2-byte rows of 1537-4096 vectors: 1024 threads, 2, 3 or 4 vectors each, dW sums in 64, 96
+    or 128 KiB of dynamic LDS; and the same rows with that switched off (sums in registers)."""
+    import ctypes
+
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=13 + cols)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    L = U.lib()
+    out = [ctypes.c_int(0) for _ in range(4)]
+    U.check(L.mg_rmsnorm_launch_info(1, cols, U.CODES[dtype], *[ctypes.byref(o) for o in out]))
+    assert [o.value for o in out] == [0, 1024, 2 if cols <= 16384 else (3 if cols <= 24576 else 4), 1024]
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    for lds in (-1, 0):
+        U.check(L.mg_set_option(b"bwd_lds", lds))
+        try:
+            dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+        finally:
+            U.check(L.mg_set_option(b"bwd_lds", -1))
+        U.assert_matches(dx, dx_ref, dtype, f"dx bwd_lds={lds}", floor=floor)
+        U.assert_dw(dw, dw_ref)
+        assert torch.isfinite(part).all(), "padding columns of a partial row were left unwritten"
+
+
 @pytest.mark.parametrize("tpr", [64, 128, 256, 512, 1024])
 def test_every_forward_workgroup_shape(tpr):
     rows, cols = 333, 4096
