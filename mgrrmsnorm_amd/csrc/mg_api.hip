@@ -152,15 +152,17 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         for (int b : {block, 512, 1024})
             if (bwd_cfg_ok(esize, tpr, need, b)) { *cfg = {kVec, tpr, need, b}; return true; }
     }
-    // 2-byte rows of 1537-4096 vectors: 1024 threads with the dW sums in LDS ("bwd_lds" = 0: in
-    // registers; 1 = from 1025 vectors on).  Beyond 2048 vectors the register kernel needs 5-8
-    // vectors per thread at 512 threads and spills (20480 bf16 columns: 4.8 -> 5.9 TB/s,
-    // 32768: 1.2 -> 5.8); at 1537-2048 vectors two such workgroups share a compute unit and
-    // gain 1-5 % (16384 x 16384: 5.77 -> 6.02 TB/s; 65536 x 16384: 5.83 -> 5.87); below that
-    // the register kernel is as fast or faster (10240 columns: 6.0 against 5.8).
+    // Rows of 2049-4096 vectors, and 2-byte rows from 1537 vectors on: 1024 threads with the dW
+    // sums in LDS ("bwd_lds" = 0: in registers; 1 = from 1025 vectors on).  Beyond 2048 vectors
+    // the register kernel needs 5-8 vectors per thread at 512 threads; with 8 sums per vector
+    // (2-byte types) it spills (20480 bf16 columns: 4.8 -> 5.9 TB/s, 32768: 1.2 -> 5.8), with 4
+    // (fp32) it merely runs 3-6 % slower (16384 columns: 5.96 -> 6.18 TB/s, 10240: 5.79 -> 6.16).
+    // At 1537-2048 vectors of a 2-byte type two such workgroups share a compute unit and gain
+    // 1-5 % (16384 x 16384: 5.77 -> 5.98 TB/s); below that, and for fp32 up to 2048 vectors,
+    // the register kernel is as fast or faster (10240 bf16 columns: 6.0 against 5.8).
     if (tpr == 0 && block == 0 && opt_bwd_lds.load() != 0) {
         const int need = ceil_div(nvec, 1024);
-        if (bwd_lds_ok(esize, nvec, need) && (nvec > 1536 || opt_bwd_lds.load() == 1)) {
+        if (bwd_lds_ok(esize, nvec, need) && (nvec > 2048 || (nvec > 1536 && esize == 2) || opt_bwd_lds.load() == 1)) {
             *cfg = {kVec, 1024, need, 1024, kFamilyLdsSums};
             return true;
         }
@@ -329,7 +331,7 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
         // one vector per lane leaves half the bytes in flight: a second workgroup makes up for it
         if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
         if (cfg.family == kFamilyGroups) { rg = (cfg.block / cfg.tpr) * cfg.items; dflt_per_cu = 1; }
-        if (cfg.family == kFamilyLdsSums) dflt_per_cu = cfg.items == 2 ? 2 : 1;   // 64, 96 or 128 KiB of LDS each
+        if (cfg.family == kFamilyLdsSums) dflt_per_cu = (es == 2 && cfg.items == 2) ? 2 : 1;   // 32-128 KiB of LDS each
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;

@@ -21,11 +21,11 @@ constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
 // per wave in flight ("row groups"); `tpr` is then a power of two from 1 to 64 and at least the
 // row's vectors (below 8 lanes per row only with 2 or 4 groups).
 constexpr int kFamilyGroups = 2;
-// Backward only: 2-byte rows of 1025-4096 vectors on 1024 threads with 2, 3 or 4 vectors each
-// and the dW sums in LDS (64, 96 or 128 KiB of dynamic LDS).
+// Backward only: rows of 1025-4096 vectors on 1024 threads with 2, 3 or 4 vectors each and the
+// dW sums in LDS (32 KiB of dynamic LDS per vector of a thread for the 2-byte types, 16 KiB for fp32).
 constexpr int kFamilyLdsSums = 3;
 constexpr bool bwd_lds_ok(int esize, long nvec, int items) {
-    return esize == 2 && nvec > 1024 && nvec <= 4096 && (items == 2 || items == 3 || items == 4) && nvec <= 1024L * items;
+    return (esize == 2 || esize == 4) && nvec > 1024 && nvec <= 4096 && (items == 2 || items == 3 || items == 4) && nvec <= 1024L * items;
 }
 constexpr bool groups_ok(long row_bytes, int tpr, int groups) {
     const bool lanes = tpr == 1 || tpr == 2 || tpr == 4 || tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64;

@@ -35,7 +35,7 @@ hipError_t run(const BwdArgs& a, hipStream_t s) {
 // dW sums in LDS: more dynamic LDS than the 64 KiB a kernel gets without asking
 template <int ITEMS>
 hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
-    if constexpr (sizeof(elem_t) == 2) {
+    if constexpr (sizeof(elem_t) == 2 || sizeof(elem_t) == 4) {
         constexpr int kLdsBytes = ITEMS * 1024 * (kVec / (int)sizeof(elem_t)) * 4;
         auto kernel = rmsnorm_bwd_rows_lds<elem_t, ITEMS>;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -797,14 +797,15 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
 }
 
 // =================================================================================
-// Backward pass 1 for 2-byte rows of 1537-4096 vectors (12 296 ... 32 768 columns): the same
-// persistent scheme with one row slot per 1024-thread workgroup, but the dW sums -- 8 floats
-// per vector, which registers no longer hold next to the row itself once a thread has more
-// than two vectors (with 5-8 vectors per thread at 512 threads the register kernel spills:
-// 4.8 TB/s at 20 480 columns, 1.2 at 32 768) -- live in LDS.  Each thread owns fixed 16-byte
-// slices of it, so no synchronisation is needed.
-//   block = TPR = 1024 threads; grid = P workgroups, one per compute unit (two with 2 vectors);
-//   dynamic LDS = ITEMS * 1024 * (16 / sizeof(T)) floats (64, 96 or 128 KiB)
+// Backward pass 1 for rows of up to 4096 vectors on 1024 threads (used from 2049 vectors on,
+// and from 1537 for the 2-byte types): the same persistent scheme with one row slot per
+// workgroup, but the dW sums -- 8 floats per vector of a 2-byte type, which registers no
+// longer hold next to the row itself once a thread has more than two vectors (with 5-8
+// vectors per thread at 512 threads the register kernel spills: 4.8 TB/s at 20 480 bf16
+// columns, 1.2 at 32 768) -- live in LDS.  Each thread owns fixed 16-byte slices of it, so no
+// synchronisation is needed.
+//   block = TPR = 1024 threads; grid = P workgroups, one per compute unit (two for 2 vectors of
+//   a 2-byte type); dynamic LDS = ITEMS * 1024 * (16 / sizeof(T)) floats (32 ... 128 KiB)
 // =================================================================================
 template <typename T, int ITEMS>
 __global__ void __launch_bounds__(1024)

@@ -190,7 +190,7 @@ def _launch_info(lib, backward, cols, dtype):
     # fp32: 4 elements per vector, any width is 4-byte aligned
     (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
     (33, 0, (0, 8, 2, 256), (0, 8, 2, 512)),            # 132 bytes: 9 vectors would idle 7 of 16 lanes
-    (16384, 0, (0, 1024, 4, 1024), (0, 512, 8, 512)),
+    (16384, 0, (0, 1024, 4, 1024), (0, 1024, 4, 1024)),   # backward: the dW sums in LDS
 ])
 def test_launch_shapes(lib, cols, dtype, fwd, bwd):
     assert _launch_info(lib, 0, cols, dtype) == fwd

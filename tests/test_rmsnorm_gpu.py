@@ -499,12 +499,14 @@ def test_row_groups_can_be_switched_off():
     U.assert_dw(dw, dw_ref)
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
-@pytest.mark.parametrize("rows,cols", [(33, 12296), (600, 16384), (21, 16383), (33, 16392), (300, 20480), (41, 24576),
-                                       (19, 32768), (7, 32767), (5, 28001)])
+@pytest.mark.parametrize("dtype,rows,cols", [(d, r, c) for d in ("bf16", "fp16") for r, c in
+                                             [(33, 12296), (600, 16384), (21, 16383), (33, 16392), (300, 20480),
+                                              (41, 24576), (19, 32768), (7, 32767), (5, 28001)]]
+                         + [("fp32", 33, 8196), ("fp32", 300, 10240), ("fp32", 41, 12288), ("fp32", 19, 16384),
+                            ("fp32", 7, 14001)])
 def test_backward_with_the_dw_sums_in_lds(dtype, rows, cols):
-    """2-byte rows of 1537-4096 vectors: 1024 threads, 2, 3 or 4 vectors each, dW sums in 64, 96
-    or 128 KiB of dynamic LDS; and the same rows with that switched off (sums in registers)."""
+    """Rows of 2049-4096 vectors (2-byte types: from 1537): 1024 threads, 2, 3 or 4 vectors each,
+    dW sums in dynamic LDS; and the same rows with that switched off (sums in registers)."""
     import ctypes
 
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=13 + cols)
@@ -513,7 +515,8 @@ def test_backward_with_the_dw_sums_in_lds(dtype, rows, cols):
     L = U.lib()
     out = [ctypes.c_int(0) for _ in range(4)]
     U.check(L.mg_rmsnorm_launch_info(1, cols, U.CODES[dtype], *[ctypes.byref(o) for o in out]))
-    assert [o.value for o in out] == [0, 1024, 2 if cols <= 16384 else (3 if cols <= 24576 else 4), 1024]
+    nvec = -(-cols * (4 if dtype == "fp32" else 2) // 16)
+    assert [o.value for o in out] == [0, 1024, -(-nvec // 1024), 1024]
     _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
     for lds in (-1, 0):
         U.check(L.mg_set_option(b"bwd_lds", lds))
