@@ -103,6 +103,9 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype,
  * overrides of megagemm_hip_tuning.h, if a process sets any: results are bit-identical from
  * run to run.  With rows == 0 the workspace is zero-filled.
  * Limits as for mg_rmsnorm_fwd (the reference caps cols at 16384 / 32768).
+ * Rows of more than 32 KiB (2-byte types: more than 24 KiB) use a kernel with more than
+ * 64 KiB of dynamic LDS, for which the library asks once per GPU on the first such call
+ * (hipFuncSetAttribute): make that call before the first stream capture rather than inside it.
  */
 int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, const void* w,
                    const float* inv_rms, int64_t rows, int64_t cols, int dtype,

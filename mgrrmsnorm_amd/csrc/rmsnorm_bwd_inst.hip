@@ -1,5 +1,7 @@
 // RMSNorm backward (pass 1) launchers for one element type; compile with
 // -DMG_DTYPE=0|1|2 (fp32 | fp16 | bf16).
+#include <atomic>
+
 #include "mg_launch.hpp"
 #include "rmsnorm_kernels.hpp"
 
@@ -38,9 +40,17 @@ hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
     if constexpr (sizeof(elem_t) == 2 || sizeof(elem_t) == 4) {
         constexpr int kLdsBytes = ITEMS * 1024 * (kVec / (int)sizeof(elem_t)) * 4;
         auto kernel = rmsnorm_bwd_rows_lds<elem_t, ITEMS>;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           kLdsBytes);
+        // asked for once per device (the first call on a device should not sit inside a stream capture)
+        static std::atomic<bool> allowed[64];
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
         if (e != hipSuccess) return e;
+        if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    kLdsBytes);
+            if (e != hipSuccess) return e;
+            if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
+        }
         kernel<<<dim3((unsigned)a.num_partials), dim3(1024), kLdsBytes, s>>>(
             (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
             a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);

@@ -317,10 +317,10 @@ def test_runs_on_the_stream_it_is_given():
     assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1)
 
 
-def test_graph_capture_and_replay():
+@pytest.mark.parametrize("rows,cols", [(1024, 4096), (300, 20480)])   # the second: backward with its dW sums in dynamic LDS
+def test_graph_capture_and_replay(rows, cols):
     """Forward, backward and the dW reduction captured in one HIP graph; every replay, with
     eager work and synchronisation in between, must reproduce the eager result."""
-    rows, cols = 1024, 4096
     dtype, code = "bf16", 2
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=31)
     xd, dyd, wd = _dev(x, dy, w)
