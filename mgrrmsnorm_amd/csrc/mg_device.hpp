@@ -112,6 +112,30 @@ __device__ __forceinline__ void load_row(Words<NW> (&v)[ITEMS], rsrc_t r, int li
     }
 }
 
+// The same in two steps, for rows that are requested long before they are used (the next
+// row of a persistent kernel): request_row() issues the loads and leaves the tail element in
+// `tail_bits` untouched; patch_row_tail() puts it into its word when the row is used, so that
+// no wait for the loads sits between the request and the work it is meant to overlap.
+template <int NW, int ITEMS, int TPR, int POLICY>
+__device__ __forceinline__ void request_row(Words<NW> (&v)[ITEMS], u32& tail_bits, rsrc_t r, int lir, const RowTail& t) {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) v[i] = buf_load<NW, POLICY>(r, (u32)(lir + i * TPR) * (NW * 4));
+    tail_bits = 0;
+    if (t.any)   // uniform over the launch; lanes that do not own the tail ask for nothing
+        tail_bits = __builtin_amdgcn_raw_buffer_load_b16(r, (int)(lir == t.lane ? t.off : 0xFFFFFFF0u), 0, POLICY);
+}
+
+template <int NW, int ITEMS>
+__device__ __forceinline__ void patch_row_tail(Words<NW> (&v)[ITEMS], u32 tail_bits, int lir, const RowTail& t) {
+    if (t.any) {
+#pragma unroll
+        for (int i = 0; i < ITEMS; ++i)
+#pragma unroll
+            for (int j = 0; j < NW; ++j)
+                v[i].v[j] = (lir == t.lane && i == t.item && j == t.word) ? tail_bits : v[i].v[j];
+    }
+}
+
 // Store vector `i` of this lane; the owner of the half-dword tail also stores that element.
 template <int NW, int TPR, int POLICY>
 __device__ __forceinline__ void store_item(rsrc_t r, int lir, int i, const Words<NW>& w, const RowTail& t) {

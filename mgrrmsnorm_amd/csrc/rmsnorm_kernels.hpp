@@ -58,8 +58,11 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
     const RowTail tail = row_tail<T, TPR>(cols, row_bytes);
     Words<NW> xv[ITEMS];
     Words<NW> wv[ITEMS];
-    load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
-    load_row<NW, ITEMS, TPR, kKeep>(wv, rw, lir, tail);
+    u32 x_tail, w_tail;
+    request_row<NW, ITEMS, TPR, kStream>(xv, x_tail, rx, lir, tail);
+    request_row<NW, ITEMS, TPR, kKeep>(wv, w_tail, rw, lir, tail);
+    patch_row_tail<NW, ITEMS>(xv, x_tail, lir, tail);
+    patch_row_tail<NW, ITEMS>(wv, w_tail, lir, tail);
 
     float ss = 0.0f;
 #pragma unroll
@@ -677,6 +680,7 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
     load_row<NW, ITEMS, TPR, kKeep>(wv, make_rsrc(w, row_bytes), lir, tail);
 
     Words<NW> xv[ITEMS], gv[ITEMS];
+    u32 x_tail, g_tail;   // the odd last element of a 2-byte row, patched in when the row is used
     long row = slot;
     bool live = row < rows;
     float s = 0.0f;
@@ -684,8 +688,8 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
         const long base = live ? row * (long)cols : 0;
         const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
         const rsrc_t rg_ = make_rsrc(dy + base, live ? row_bytes : 0u);
-        load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
-        load_row<NW, ITEMS, TPR, kStream>(gv, rg_, lir, tail);
+        request_row<NW, ITEMS, TPR, kStream>(xv, x_tail, rx, lir, tail);
+        request_row<NW, ITEMS, TPR, kStream>(gv, g_tail, rg_, lir, tail);
         if (live) s = inv_rms[row];
     }
 
@@ -693,16 +697,19 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
         const long nrow = row + nslots;
         const bool nlive = nrow < rows;
         Words<NW> nxv[PREFETCH ? ITEMS : 1], ngv[PREFETCH ? ITEMS : 1];
+        u32 nx_tail = 0, ng_tail = 0;
         float ns = 0.0f;
         if constexpr (PREFETCH) {
             // request the next row of this slot now (nothing is fetched when there is none)
             const long nbase = nlive ? nrow * (long)cols : 0;
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
-            load_row<NW, ITEMS, TPR, kStream>(nxv, rx, lir, tail);
-            load_row<NW, ITEMS, TPR, kStream>(ngv, rg_, lir, tail);
+            request_row<NW, ITEMS, TPR, kStream>(nxv, nx_tail, rx, lir, tail);
+            request_row<NW, ITEMS, TPR, kStream>(ngv, ng_tail, rg_, lir, tail);
             if (nlive) ns = inv_rms[nrow];
         }
+        patch_row_tail<NW, ITEMS>(xv, x_tail, lir, tail);
+        patch_row_tail<NW, ITEMS>(gv, g_tail, lir, tail);
 
         // A = sum dy*w*x over the row; dW += dy*x*s
         float a = 0.0f;
@@ -749,14 +756,15 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
         if constexpr (PREFETCH) {
 #pragma unroll
             for (int i = 0; i < ITEMS; ++i) { xv[i] = nxv[i]; gv[i] = ngv[i]; }
+            x_tail = nx_tail; g_tail = ng_tail;
         } else {
             // wide rows: no second copy of the row in registers; the next row is requested
             // once this one is stored, and a second workgroup on the CU covers the wait
             const long nbase = nlive ? nrow * (long)cols : 0;
             const rsrc_t rx = make_rsrc(x + nbase, nlive ? row_bytes : 0u);
             const rsrc_t rg_ = make_rsrc(dy + nbase, nlive ? row_bytes : 0u);
-            load_row<NW, ITEMS, TPR, kStream>(xv, rx, lir, tail);
-            load_row<NW, ITEMS, TPR, kStream>(gv, rg_, lir, tail);
+            request_row<NW, ITEMS, TPR, kStream>(xv, x_tail, rx, lir, tail);
+            request_row<NW, ITEMS, TPR, kStream>(gv, g_tail, rg_, lir, tail);
             if (nlive) ns = inv_rms[nrow];
         }
         row = nrow; live = nlive; s = ns;
@@ -840,8 +848,11 @@ rmsnorm_bwd_rows_lds(T* __restrict__ dx, float* __restrict__ dw_part, int ld, co
         const bool live = row < rows;
         const long base = live ? row * (long)cols : 0;
         Words<4> xv[ITEMS], gv[ITEMS];
-        load_row<4, ITEMS, TPR, kStream>(xv, make_rsrc(x + base, live ? row_bytes : 0u), tid, tail);
-        load_row<4, ITEMS, TPR, kStream>(gv, make_rsrc(dy + base, live ? row_bytes : 0u), tid, tail);
+        u32 x_tail, g_tail;
+        request_row<4, ITEMS, TPR, kStream>(xv, x_tail, make_rsrc(x + base, live ? row_bytes : 0u), tid, tail);
+        request_row<4, ITEMS, TPR, kStream>(gv, g_tail, make_rsrc(dy + base, live ? row_bytes : 0u), tid, tail);
+        patch_row_tail<4, ITEMS>(xv, x_tail, tid, tail);
+        patch_row_tail<4, ITEMS>(gv, g_tail, tid, tail);
         const float s = live ? inv_rms[row] : 0.0f;
 
         float a = 0.0f;
