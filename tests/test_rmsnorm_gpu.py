@@ -208,7 +208,9 @@ def test_non_finite_rows_behave_like_the_formula(dtype, cols):
 # --------------------------------------------------------------------------- determinism
 
 @pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 2000, 5120), ("fp32", 777, 1000),
-                                             ("bf16", 100003, 128), ("fp32", 50001, 64)])
+                                             ("bf16", 100003, 128), ("fp32", 50001, 64),
+                                             ("bf16", 100003, 80), ("fp16", 70001, 100),    # row groups, aligned and ragged
+                                             ("bf16", 3000, 16384), ("fp16", 1500, 32768), ("fp32", 1500, 12288)])  # dW sums in LDS
 def test_dw_is_bit_identical_across_runs(dtype, rows, cols):
     x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=3)
     xd, dyd, wd = _dev(x, dy, w)
@@ -250,6 +252,7 @@ FULL = [
     ("bf16", 65536, 4100), ("fp16", 65536, 4100),
     ("bf16", 65536, 5120), ("fp16", 65536, 5120),
     ("bf16", 65536, 16384), ("fp16", 65536, 16384),   # 2^31 bytes per tensor: offsets need 64 bits
+    ("fp16", 8192, 32768), ("fp32", 8192, 12288),     # backward with the dW sums in LDS: 4 and 3 vectors per thread
     ("fp32", 70000, 16388),   # 4.6 GB per tensor, rows 4-byte aligned only: offsets beyond 2^32
     ("bf16", 2097152, 128),   # rows narrower than a wave, one vector per lane: 16 rows per wave in flight
     ("bf16", 2097152, 80),    # ... at a pitch of 160 bytes
