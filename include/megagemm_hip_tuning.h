@@ -70,10 +70,16 @@ int mg_row_probe(void* dst, const void* a, const void* b, int64_t rows, int64_t 
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
  * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
- * workgroup), "bwd_wg_per_cu", "bwd_prefetch" (1/0: request the next row before reducing
+ * workgroup), "bwd_wg_per_cu", "bwd_partials" (workgroups of the persistent backward grid, which is
+ * also the number of partial rows; 0 = automatic), "bwd_prefetch" (1/0: request the next row before reducing
  * the current one; -1 = automatic), "narrow_groups" (the row-group layout for rows of at most
  * 64 vectors: 1, 2 or 4 groups in flight, 0 = never, -1 = automatic; a "fwd_tpr" / "fwd_items" /
- * "bwd_tpr" / "bwd_block" override switches the automatic choice off), "swiglu_unroll",
+ * "bwd_tpr" / "bwd_block" override switches the automatic choice off), "bwd_lds" (backward rows
+ * of 1025-4096 vectors on 1024 threads with the dW sums in LDS: 0 = never, 1 = from 1025
+ * vectors on, -1 = automatic), "bwd_ring" (backward rows at 16-byte pitches that fill their
+ * lanes at one vector per thread, kept in flight through a ring of register buffers: 0 = never,
+ * 2 or 4 = that many buffers, -1 = automatic; a "bwd_tpr" / "bwd_block" override switches it
+ * off as well), "swiglu_unroll",
  * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
  * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
  * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for

@@ -30,7 +30,7 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1}, opt_bwd_ring{-1}, opt_bwd_partials{0};
 
 // Consecutive logical workgroups one die handles at a time in the one-shot streaming
 // kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
@@ -147,6 +147,23 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
         const int nt = narrow_items(row_bytes, tpr) ? tpr : (tpr == 0 ? narrow_default_tpr(row_bytes, true) : 0);
         if (nt) { *cfg = {kVec, nt, narrow_items(row_bytes, nt), 512}; return true; }
     }
+    // Rows whose pitch is a multiple of 16 bytes and that fill at least three quarters of the lanes
+    // of 64 ... 1024 threads at one vector each: one vector per thread and a ring of register
+    // buffers ("bwd_ring" = 0: never; 2 or 4: that many buffers).  Against two vectors at half the
+    // threads with the copied prefetch (bf16, 65536 rows): 768 columns 49.4 against 50.4 us, 2048
+    // 124.3 against 129.0, 4096 250.9 against 256, 8192 at 16384 rows 126.4 against 130.0, 4096 x 4096
+    // 18.4 against 18.85.  Rows of 1025-1536 vectors (fp32: up to 2048) take two vectors on 1024
+    // threads the same way (10240 bf16 columns 161.8 against 166.2 us, 12288 195.0 against 206.0).
+    if (tpr == 0 && block == 0 && opt_bwd_ring.load() != 0 && row_bytes % kVec == 0 && nvec >= 57) {
+        if (nvec <= 1024) {
+            int t = 64;
+            while (t < nvec) t *= 2;
+            if (nvec * 4 >= 3L * t) { *cfg = {kVec, t, 1, t > 512 ? 1024 : 512, kFamilyRing, 0}; return true; }
+        } else if (nvec * 5 >= 3L * 2048 && nvec <= ((esize == 4 || opt_bwd_ring.load() == 2) ? 2048 : 1536)) {
+            *cfg = {kVec, 1024, 2, 1024, kFamilyRing, 0};
+            return true;
+        }
+    }
     if (tpr_ok(tpr)) {
         const int need = round_items(ceil_div(nvec, tpr));
         for (int b : {block, 512, 1024})
@@ -254,7 +271,7 @@ int mg_set_option(const char* key, int value) {
         {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
-        {"bwd_prefetch", &opt_bwd_prefetch},
+        {"bwd_prefetch", &opt_bwd_prefetch}, {"bwd_ring", &opt_bwd_ring}, {"bwd_partials", &opt_bwd_partials},
     };
     if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
     for (auto& t : table)
@@ -332,10 +349,12 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
         if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
         if (cfg.family == kFamilyGroups) { rg = (cfg.block / cfg.tpr) * cfg.items; dflt_per_cu = 1; }
         if (cfg.family == kFamilyLdsSums) dflt_per_cu = (es == 2 && cfg.items == 2) ? 2 : 1;   // 32-128 KiB of LDS each
+        if (cfg.family == kFamilyRing) dflt_per_cu = 1;
     }
     int per_cu = opt_bwd_wg_per_cu.load();
     if (per_cu < 1 || per_cu > 8) per_cu = dflt_per_cu;
     int64_t p = (int64_t)cus * per_cu;
+    if (opt_bwd_partials.load() > 0) p = opt_bwd_partials.load();   // "bwd_partials": that many workgroups
     const int64_t by_rows = (rows + rg - 1) / rg;
     if (p > by_rows) p = by_rows;
     if (p < 1) p = 1;
@@ -373,6 +392,21 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
     if (!generic) generic = !choose_bwd(row_bytes, es, &cfg) && !choose_streaming(row_bytes, &cfg);
+    if (!generic && cfg.family == kFamilyRing) {
+        // Two buffers (one row requested ahead) for rows that fill their lanes, four (three rows
+        // ahead) for rows that leave up to a quarter of the lanes idle (bf16, 65536 rows, two / four
+        // buffers / the copying loop: 2048 columns 126.6 / 131.1 / 127.8 us, 4096 columns 261.4 / 273.1 /
+        // 262.0, 768 columns 56.2 / 49.1 / 50.2, 3072 columns 204.5 / 192.2 / 196.2), and four as well
+        // while a slot has at most 32 rows, where filling the memory pipeline at the start counts
+        // (4096 x 4096: 19.2 / 18.8 / 18.9).  Two vectors per thread: always two buffers (registers).
+        const int forced = opt_bwd_ring.load();
+        const long nvec = (row_bytes + kVec - 1) / kVec;
+        const long slots = num_partials * (cfg.block / cfg.tpr);
+        const bool full = nvec * 8 > 7L * cfg.tpr;
+        if (cfg.items != 1) cfg.depth = 2;
+        else if (forced == 2 || forced == 4) cfg.depth = forced;
+        else cfg.depth = (!full || (rows + slots - 1) / slots <= 32) ? 4 : 2;
+    }
     const int prefetch = opt_bwd_prefetch.load();   // every option is read once per call
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for

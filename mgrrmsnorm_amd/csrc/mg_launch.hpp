@@ -14,7 +14,9 @@ struct RowCfg {
     int block;  // backward only: threads per workgroup, 1024 or 512
     int family; // kFamilyResident (rows held in registers), kFamilyStreaming (rows read twice) or
                 // kFamilyGroups (narrow rows, one vector per lane; `items` = row groups in flight) or
-                // kFamilyLdsSums (backward: rows in registers, dW sums in LDS)
+                // kFamilyLdsSums (backward: rows in registers, dW sums in LDS) or
+                // kFamilyRing (backward: a ring of `depth` register buffers per row slot)
+    int depth;  // kFamilyRing only: register buffers per row slot (2 or 4); 0 = chosen per call
 };
 constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
 // Rows of at most 64 vectors can also go one vector per lane, `items` groups of 64/tpr rows
@@ -26,6 +28,16 @@ constexpr int kFamilyGroups = 2;
 constexpr int kFamilyLdsSums = 3;
 constexpr bool bwd_lds_ok(int esize, long nvec, int items) {
     return (esize == 2 || esize == 4) && nvec > 1024 && nvec <= 4096 && (items == 2 || items == 3 || items == 4) && nvec <= 1024L * items;
+}
+// Backward only: rows whose pitch is a multiple of 16 bytes, one vector per thread on 64 ... 1024
+// threads (512-thread workgroups, 1024 for 1024 threads per row), or two vectors on 1024
+// threads, with the rows of a slot kept in flight through a ring of register buffers.
+constexpr int kFamilyRing = 4;
+constexpr bool bwd_ring_ok(long row_bytes, int tpr, int items, int depth) {
+    const long nvec = (row_bytes + 15) / 16;
+    const bool shape = (items == 1 && (tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024)) ||
+                       (items == 2 && tpr == 1024);
+    return shape && row_bytes % 16 == 0 && nvec <= (long)tpr * items && (depth == 2 || depth == 4);
 }
 constexpr bool groups_ok(long row_bytes, int tpr, int groups) {
     const bool lanes = tpr == 1 || tpr == 2 || tpr == 4 || tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64;

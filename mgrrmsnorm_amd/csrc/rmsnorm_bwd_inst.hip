@@ -60,6 +60,32 @@ hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
     }
 }
 
+template <int TPR, int ITEMS, int DEPTH>
+hipError_t run_ring(const BwdArgs& a, hipStream_t s) {
+    constexpr int BLOCK = TPR > 512 ? TPR : 512;
+    rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH><<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
+        (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+        a.rows, a.cols, 1.0f / (float)a.cols);
+    return hipGetLastError();
+}
+
+template <int TPR, int ITEMS>
+hipError_t ring_by_depth(int depth, const BwdArgs& a, hipStream_t s) {
+    return depth == 4 ? run_ring<TPR, ITEMS, 4>(a, s) : run_ring<TPR, ITEMS, 2>(a, s);
+}
+
+hipError_t ring_by_shape(const RowCfg& cfg, const BwdArgs& a, hipStream_t s) {
+    if (!bwd_ring_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items, cfg.depth)) return hipErrorInvalidValue;
+    if (cfg.items == 2) return cfg.depth == 2 ? run_ring<1024, 2, 2>(a, s) : hipErrorInvalidValue;   // four buffers would spill
+    switch (cfg.tpr) {
+        case 64: return ring_by_depth<64, 1>(cfg.depth, a, s);
+        case 128: return ring_by_depth<128, 1>(cfg.depth, a, s);
+        case 256: return ring_by_depth<256, 1>(cfg.depth, a, s);
+        case 512: return ring_by_depth<512, 1>(cfg.depth, a, s);
+        default: return ring_by_depth<1024, 1>(cfg.depth, a, s);
+    }
+}
+
 template <int TPR, int BLOCK>
 hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
     switch (items) {
@@ -169,6 +195,7 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
         if (!bwd_lds_ok((int)sizeof(elem_t), nvec, cfg.items)) return hipErrorInvalidValue;
         return cfg.items == 2 ? run_lds_sums<2>(a, s) : (cfg.items == 3 ? run_lds_sums<3>(a, s) : run_lds_sums<4>(a, s));
     }
+    if (cfg.family == kFamilyRing) return ring_by_shape(cfg, a, s);
     if (cfg.family == kFamilyGroups) {
         if (!groups_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items)) return hipErrorInvalidValue;
         switch (cfg.tpr) {

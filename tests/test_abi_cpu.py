@@ -155,11 +155,11 @@ def _launch_info(lib, backward, cols, dtype):
 
 @pytest.mark.parametrize("cols,dtype,fwd,bwd", [
     # 2-byte types: 8 elements per 16-byte vector
-    (4096, 2, (0, 256, 2, 256), (0, 256, 2, 512)),      # metric shape: one row per 256-thread workgroup
-    (2048, 1, (0, 128, 2, 256), (0, 128, 2, 512)),
+    (4096, 2, (0, 256, 2, 256), (0, 512, 1, 512)),      # metric shape: one row per 256-thread workgroup; backward one vector per thread (register ring)
+    (2048, 1, (0, 128, 2, 256), (0, 256, 1, 512)),
     (4100, 2, (0, 256, 3, 256), (0, 512, 2, 512)),      # 513 vectors: 3 per thread rather than 2 half-empty
     (5120, 1, (0, 512, 2, 512), (0, 512, 2, 512)),
-    (8192, 2, (0, 512, 2, 512), (0, 512, 2, 512)),
+    (8192, 2, (0, 512, 2, 512), (0, 1024, 1, 1024)),
     (16384, 2, (0, 1024, 2, 1024), (0, 1024, 2, 1024)),
     (4099, 2, (0, 256, 3, 256), (0, 512, 2, 512)),      # odd width of a 2-byte type: same kernels, one lane moves the last element
     (100000, 1, (0, 1024, 0, 1024), (0, 1024, 0, 1024)),  # wider than registers hold: 1024 threads stream the row twice
@@ -179,8 +179,8 @@ def _launch_info(lib, backward, cols, dtype):
     # 8, 16 or 32 lanes per row; forward up to 4 vectors per lane (128 vectors), backward up to 2 (56)
     (256, 1, (0, 8, 4, 256), (0, 16, 2, 512)),
     (512, 2, (0, 16, 4, 256), (0, 64, 1, 512)),         # 64 vectors: backward takes one wave per row
-    (768, 2, (0, 32, 3, 256), (0, 64, 2, 512)),
-    (1024, 1, (0, 32, 4, 256), (0, 64, 2, 512)),
+    (768, 2, (0, 32, 3, 256), (0, 128, 1, 512)),         # 96 vectors fill three quarters of 128 lanes
+    (1024, 1, (0, 32, 4, 256), (0, 128, 1, 512)),
     (1032, 2, (0, 64, 3, 256), (0, 128, 2, 512)),        # 129 vectors: one wave per row
     (1000, 2, (0, 64, 2, 256), (0, 128, 1, 512)),        # 125 vectors, pitch 2000 bytes: contiguous pieces per instruction
     # ragged rows that leave too many lanes idle, or are long, keep several vectors per lane
@@ -188,13 +188,28 @@ def _launch_info(lib, backward, cols, dtype):
     (299, 1, (0, 16, 3, 256), (0, 16, 3, 512)),         # 598 bytes, rows only 2-byte aligned
     (999, 1, (0, 64, 2, 256), (0, 64, 2, 512)),         # 1998 bytes
     # fp32: 4 elements per vector, any width is 4-byte aligned
-    (4096, 0, (0, 512, 2, 512), (0, 512, 2, 512)),
+    (4096, 0, (0, 512, 2, 512), (0, 1024, 1, 1024)),
+    (8192, 0, (0, 1024, 2, 1024), (0, 1024, 2, 1024)),  # 2048 vectors: two per thread, still a register ring
+    (12288, 2, (0, 512, 3, 512), (0, 1024, 2, 1024)),
     (33, 0, (0, 8, 2, 256), (0, 8, 2, 512)),            # 132 bytes: 9 vectors would idle 7 of 16 lanes
     (16384, 0, (0, 1024, 4, 1024), (0, 1024, 4, 1024)),   # backward: the dW sums in LDS
 ])
 def test_launch_shapes(lib, cols, dtype, fwd, bwd):
     assert _launch_info(lib, 0, cols, dtype) == fwd
     assert _launch_info(lib, 1, cols, dtype) == bwd
+
+
+def test_ring_option_switches_the_backward_layout(lib):
+    """"bwd_ring" = 0 gives back two vectors per thread at half the threads; -1 is automatic."""
+    try:
+        assert lib.mg_set_option(b"bwd_ring", 0) == 0
+        assert _launch_info(lib, 1, 4096, 2) == (0, 256, 2, 512)
+        assert _launch_info(lib, 1, 8192, 2) == (0, 512, 2, 512)
+    finally:
+        assert lib.mg_set_option(b"bwd_ring", -1) == 0
+    assert _launch_info(lib, 1, 4096, 2) == (0, 512, 1, 512)
+    # rows whose pitch is not a multiple of 16 bytes never take the ring
+    assert _launch_info(lib, 1, 4100, 2) == (0, 512, 2, 512)
 
 
 def test_launch_info_rejects_bad_arguments(lib):
@@ -209,8 +224,10 @@ def test_set_option(lib):
     assert lib.mg_set_option(b"no_such_key", 1) == -1 and "unknown key" in _err(lib)
     assert lib.mg_set_option(None, 1) == -1
     for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_block", b"bwd_wg_per_cu", b"swiglu_unroll",
-                b"force_generic"):
+                b"force_generic", b"bwd_partials"):
         assert lib.mg_set_option(key, 0) == 0
+    for key in (b"bwd_ring", b"bwd_lds", b"bwd_prefetch", b"narrow_groups", b"xcd_group"):
+        assert lib.mg_set_option(key, -1) == 0
 
 
 def test_fastdiv_matches_integer_division(tmp_path):

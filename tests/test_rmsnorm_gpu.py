@@ -502,6 +502,43 @@ def test_row_groups_can_be_switched_off():
     U.assert_dw(dw, dw_ref)
 
 
+@pytest.mark.parametrize("dtype,rows,cols,shape", [
+    ("bf16", 300, 4096, (512, 1, 512)), ("bf16", 4096, 4096, (512, 1, 512)), ("fp16", 77, 768, (128, 1, 512)),
+    ("bf16", 20000, 512, (64, 1, 512)), ("fp16", 1000, 2048, (256, 1, 512)), ("bf16", 530, 8192, (1024, 1, 1024)),
+    ("bf16", 64, 12288, (1024, 2, 1024)), ("bf16", 700, 10240, (1024, 2, 1024)), ("fp32", 33, 8192, (1024, 2, 1024)),
+    ("fp32", 1500, 1024, (256, 1, 512)), ("fp32", 259, 3072, (1024, 1, 1024)), ("bf16", 3, 6144, (1024, 1, 1024)),
+    ("fp16", 513, 1000, (128, 1, 512))])
+def test_backward_over_a_ring_of_register_buffers(dtype, rows, cols, shape):
+    """Rows at 16-byte pitches that fill their lanes: one vector per thread (two on 1024 threads
+    beyond 1024 vectors), rows kept in flight through 2 or 4 register buffers.  Both depths must
+    agree bit for bit (same layout, same order of every sum) and meet the oracle; with the ring
+    switched off the copying loop runs instead and meets the oracle as well."""
+    import ctypes
+
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=31 + cols)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    L = U.lib()
+    out = [ctypes.c_int(0) for _ in range(4)]
+    U.check(L.mg_rmsnorm_launch_info(1, cols, U.CODES[dtype], *[ctypes.byref(o) for o in out]))
+    assert tuple(o.value for o in out[1:]) == shape
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    got = {}
+    for ring in (-1, 2, 4, 0):
+        U.check(L.mg_set_option(b"bwd_ring", ring))
+        try:
+            dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+        finally:
+            U.check(L.mg_set_option(b"bwd_ring", -1))
+        U.assert_matches(dx, dx_ref, dtype, f"dx bwd_ring={ring}", floor=floor)
+        U.assert_dw(dw, dw_ref)
+        assert torch.isfinite(part).all(), "padding columns of a partial row were left unwritten"
+        got[ring] = (dx.clone(), dw.clone())
+    for ring in (2, 4):
+        assert torch.equal(got[ring][0].view(torch.uint8), got[-1][0].view(torch.uint8)), f"dx differs at depth {ring}"
+        assert torch.equal(got[ring][1].view(torch.uint8), got[-1][1].view(torch.uint8)), f"dW differs at depth {ring}"
+
+
 @pytest.mark.parametrize("dtype,rows,cols", [(d, r, c) for d in ("bf16", "fp16") for r, c in
                                              [(33, 12296), (600, 16384), (21, 16383), (33, 16392), (300, 20480),
                                               (41, 24576), (19, 32768), (7, 32767), (5, 28001)]]
