@@ -418,21 +418,37 @@ def time_configs(lib):
 
     out = {}
     for name in CONFIGS:
-        wl = make_workload(lib, name, nsets=0)
-        big = wl.step_bytes > 1e9
-        rec = {}
-        for kname, nbytes in wl.kernels.items():
-            t = time_kernel(wl, kname, launches=20 if big else 100)
-            short = kname.split("_")[-1]
-            rec[short + "_us"] = round(t * 1e6, 2)
-            rec[short + "_GB/s"] = round(nbytes / t / 1e9)
-        # the plain streaming probe on the same tensors: one read + one write, two reads + one write
-        kinds = ["copy"] + (["2r1w"] if getattr(wl, "backward", True) else [])
-        for kind in kinds:
-            t = time_kernel(wl, None, launches=20 if big else 100, fn=lambda i, st: wl.probe(kind, i, st))
-            rec["probe_" + kind + "_GB/s"] = round((2 if kind == "copy" else 3) * wl.tensor_bytes / t / 1e9)
-        out[name] = rec
-        log(f"[bench] config {name}: {rec}")
+        wl = None
+        try:
+            wl = make_workload(lib, name, nsets=0)
+            big = wl.step_bytes > 1e9
+            n_launch = 20 if big else 100
+            rec = {}
+            for kname, nbytes in wl.kernels.items():
+                t = time_kernel(wl, kname, launches=n_launch)
+                short = kname.split("_")[-1]
+                rec[short + "_us"] = round(t * 1e6, 2)
+                rec[short + "_GB/s"] = round(nbytes / t / 1e9)
+            # the plain streaming probe on the same tensors: one read + one write, two reads + one write
+            kinds = ["copy"] + (["2r1w"] if getattr(wl, "backward", True) else [])
+            for kind in kinds:
+                t = time_kernel(wl, None, launches=n_launch, fn=lambda i, st: wl.probe(kind, i, st))
+                rec["probe_" + kind + "_GB/s"] = round((2 if kind == "copy" else 3) * wl.tensor_bytes / t / 1e9)
+            # the same bytes moved by whole rows (a workgroup per row forward, a persistent grid of one
+            # workgroup per compute unit backward): what whole-row ownership costs at this row length
+            rb = getattr(wl, "row_bytes", 0)
+            if rb and rb % 16 == 0 and rb <= 65536:
+                t = time_kernel(wl, None, launches=n_launch, fn=lambda i, st: wl.probe("rows_copy", i, st))
+                rec["probe_rows_copy_GB/s"] = round(2 * wl.tensor_bytes / t / 1e9)
+                if getattr(wl, "backward", False):
+                    cus = torch.cuda.get_device_properties(0).multi_processor_count
+                    t = time_kernel(wl, None, launches=n_launch, fn=lambda i, st: wl.probe(("rows_2r1w", cus), i, st))
+                    rec["probe_rows_2r1w_GB/s"] = round(3 * wl.tensor_bytes / t / 1e9)
+            out[name] = rec
+            log(f"[bench] config {name}: {rec}")
+        except Exception as exc:     # noqa: BLE001 -- one configuration must not cost the others
+            out[name] = {"error": f"{type(exc).__name__}: {exc}"}
+            log(f"[bench] config {name} failed: {out[name]['error']}")
         del wl
         gc.collect()
         torch.cuda.empty_cache()
@@ -598,24 +614,9 @@ def main():
     sec_per_step = wall[mode] / args.steps
     value = wl.step_bytes / sec_per_step / 1e9
 
-    kern = {}
-    for name, nbytes in wl.kernels.items():
-        t = time_kernel(wl, name)
-        kern[name] = {"us": round(t * 1e6, 3), "GB/s": round(nbytes / t / 1e9, 1), "bytes": nbytes}
-        log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch, {nbytes / t / 1e9:.0f} GB/s")
-    for name in getattr(wl, "extra_kernels", []):
-        t = time_kernel(wl, name)
-        kern[name] = {"us": round(t * 1e6, 3)}
-        log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch")
-    dom = wl.dominant
-    achieved = kern[dom]["GB/s"]
-    traffic, traffic_source = committed_traffic(dom, wl.name)
-    roofline = {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                "algorithmic_bytes": kern[dom]["bytes"], "avg_launch_us": kern[dom]["us"]}
-    ceil = ceiling(wl)
-    log(f"[bench] ceiling on the same tensors: {ceil}")
-
+    # The headline figures are fixed from here on; everything below adds detail to the same JSON
+    # line, and a failure in one of those sections is recorded under its key instead of losing
+    # the line.
     out = {
         "metric": "RMSNorm fwd+bwd HBM GB/s at [4096x4096] bf16" if wl.name == "rmsnorm_fwd_bwd_4096x4096_bf16"
                   else f"{wl.name} HBM GB/s",
@@ -625,24 +626,57 @@ def main():
         "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
         "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
         "readings_us_per_step": {m: [round(t / args.steps * 1e6, 3) for t in r] for m, r in readings.items()},
-        "kernels": kern, "roofline": roofline, "ceiling": ceil, "library_source_sha16": library_source_sha16(),
+        "library_source_sha16": library_source_sha16(),
     }
-    if isinstance(wl, RmsNormWorkload) and (args.surface == "module" or not args.no_configs):
-        out["module"] = time_module_surface(wl.rows, wl.cols, wl.dtype)
-        log(f"[bench] nn.Module surface: {out['module']}")
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl)
-        log(f"[bench] cpu baseline: {out['cpu_baseline']}")
-    del wl
-    import gc
 
-    gc.collect()
-    torch.cuda.empty_cache()
-    if not args.no_configs:
-        out["configs"] = time_configs(lib)
-    if args.sweep:
-        out["sweep"] = sweep(lib)
-    print(json.dumps(out), flush=True)
+    def section(key, fn):
+        try:
+            out[key] = fn()
+        except Exception as exc:     # noqa: BLE001 -- recorded, the line is still printed
+            out[key] = {"error": f"{type(exc).__name__}: {exc}"}
+            log(f"[bench] section '{key}' failed: {out[key]['error']}")
+            try:
+                torch.cuda.synchronize()
+            except Exception:        # noqa: BLE001
+                pass
+        return out[key]
+
+    def kernels_and_roofline():
+        kern = {}
+        for name, nbytes in wl.kernels.items():
+            t = time_kernel(wl, name)
+            kern[name] = {"us": round(t * 1e6, 3), "GB/s": round(nbytes / t / 1e9, 1), "bytes": nbytes}
+            log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch, {nbytes / t / 1e9:.0f} GB/s")
+        for name in getattr(wl, "extra_kernels", []):
+            t = time_kernel(wl, name)
+            kern[name] = {"us": round(t * 1e6, 3)}
+            log(f"[bench] kernel {name}: {t * 1e6:.2f} us/launch")
+        out["kernels"] = kern
+        dom = wl.dominant
+        achieved = kern[dom]["GB/s"]
+        traffic, traffic_source = committed_traffic(dom, wl.name)
+        return {"bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                "algorithmic_bytes": kern[dom]["bytes"], "avg_launch_us": kern[dom]["us"]}
+
+    try:
+        section("roofline", kernels_and_roofline)
+        log(f"[bench] ceiling on the same tensors: {section('ceiling', lambda: ceiling(wl))}")
+        if isinstance(wl, RmsNormWorkload) and (args.surface == "module" or not args.no_configs):
+            log(f"[bench] nn.Module surface: {section('module', lambda: time_module_surface(wl.rows, wl.cols, wl.dtype))}")
+        if not args.no_cpu_baseline:
+            log(f"[bench] cpu baseline: {section('cpu_baseline', lambda: cpu_baseline(wl))}")
+        del wl
+        import gc
+
+        gc.collect()
+        torch.cuda.empty_cache()
+        if not args.no_configs:
+            section("configs", lambda: time_configs(lib))
+        if args.sweep:
+            section("sweep", lambda: sweep(lib))
+    finally:
+        print(json.dumps(out), flush=True)
 
 
 if __name__ == "__main__":

@@ -127,6 +127,16 @@ def build(jobs: int | None = None, verbose: bool = False, binding: bool = True, 
     return lib_path
 
 
+def is_current() -> bool:
+    """True when both built files exist and are newer than every source they are made from
+    (csrc/*.hip, *.hpp, *.cpp, include/*.h and this recipe)."""
+    outs = [LIB_PATH, BINDING_PATH]
+    if not all(p.exists() for p in outs):
+        return False
+    srcs = [*CSRC.glob("*.hip"), *CSRC.glob("*.hpp"), *CSRC.glob("*.cpp"), *INCLUDE.glob("*.h"), Path(__file__)]
+    return min(p.stat().st_mtime for p in outs) >= max(p.stat().st_mtime for p in srcs)
+
+
 if __name__ == "__main__":
     path = build(verbose="-v" in sys.argv, binding="--no-binding" not in sys.argv)
     print(f"built {path}" + ("" if "--no-binding" in sys.argv else f" and {BINDING_PATH}"))

@@ -239,13 +239,8 @@ int check_rmsnorm_dims(const char* fn, int64_t rows, int64_t cols, int dtype) {
     return MG_OK;
 }
 
-// The launchers report hipGetLastError() after <<<>>>; an error that another HIP user left
-// on this thread earlier would be taken for ours, so it is dropped before we launch.
-void drop_stale_error() { (void)hipGetLastError(); }
-
 template <typename F32, typename F16, typename BF16>
 hipError_t by_dtype(int dtype, F32 f32, F16 f16, BF16 bf16) {
-    drop_stale_error();
     switch (dtype) {
         case MG_F32: return f32();
         case MG_F16: return f16();
@@ -377,8 +372,7 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: dw_partial must be a 16-byte aligned device pointer");
     hipStream_t s = (hipStream_t)stream;
     if (rows == 0) {
-        drop_stale_error();
-        hipError_t e = launch_fill_zero(dw_partial, (long)(num_partials * ld), s);
+            hipError_t e = launch_fill_zero(dw_partial, (long)(num_partials * ld), s);
         if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd: zero fill", e);
         return MG_OK;
     }
@@ -438,7 +432,6 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: dw_partial must be a 16-byte aligned device pointer");
     if (!aligned(dw_f32, 4) || (dw_cast != nullptr && !aligned(dw_cast, esize_of(cast_dtype))))
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_dw_reduce: an output pointer is not aligned to its element size");
-    drop_stale_error();
     hipError_t e = launch_dw_reduce(dw_f32, dw_cast, cast_dtype, dw_partial, (int)num_partials, (int)ld, (int)cols,
                                     (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_rmsnorm_dw_reduce: launch", e);
@@ -500,7 +493,6 @@ int mg_copy_bytes(void* dst, const void* src, int64_t bytes, void* stream) {
     if (bytes == 0) return MG_OK;
     if (dst == nullptr || src == nullptr || !aligned(dst, 16) || !aligned(src, 16))
         return fail(MG_ERR_INVALID_ARG, "mg_copy_bytes: dst and src must be 16-byte aligned device pointers");
-    drop_stale_error();
     hipError_t e = launch_copy(dst, src, (long)bytes, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_copy_bytes: launch", e);
     return MG_OK;
@@ -513,7 +505,6 @@ int mg_stream_probe(void* dst, const void* a, const void* b, int64_t bytes, void
     if (bytes == 0) return MG_OK;
     if (dst == nullptr || a == nullptr || !aligned(dst, 4) || !aligned(a, 4) || !aligned(b, 4))
         return fail(MG_ERR_INVALID_ARG, "mg_stream_probe: dst, a (and b, if given) must be 4-byte aligned device pointers");
-    drop_stale_error();
     hipError_t e = launch_stream_probe(dst, a, b, (long)bytes, xcd_group_or(kXcdGroupStreaming), (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_stream_probe: launch", e);
     return MG_OK;
@@ -531,7 +522,6 @@ int mg_row_probe(void* dst, const void* a, const void* b, int64_t rows, int64_t 
     if (rows == 0) return MG_OK;
     if (dst == nullptr || a == nullptr || !aligned(dst, 4) || !aligned(a, 4) || !aligned(b, 4))
         return fail(MG_ERR_INVALID_ARG, "mg_row_probe: dst, a (and b, if given) must be 4-byte aligned device pointers");
-    drop_stale_error();
     hipError_t e = launch_row_probe(dst, a, b, (long)rows, (long)row_bytes, (long)workgroups, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_row_probe: launch", e);
     return MG_OK;
@@ -573,7 +563,6 @@ int mg_swiglu_fwd(void* h, const void* gu, int64_t M, int64_t H, int dtype, void
     if (!aligned(h, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_fwd: a pointer is not aligned to its element size");
     const int mode = swiglu_mode(H * es, aligned(h, 16) && aligned(gu, 16));
-    drop_stale_error();
     hipError_t e = launch_swiglu_fwd(dtype, mode, swiglu_unroll(1, 8), xcd_group_or(kXcdGroupStreaming), h, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_fwd: launch", e);
     return MG_OK;
@@ -589,7 +578,6 @@ int mg_swiglu_bwd(void* dgu, const void* dh, const void* gu, int64_t M, int64_t 
     if (!aligned(dgu, es) || !aligned(dh, es) || !aligned(gu, es))
         return fail(MG_ERR_INVALID_ARG, "mg_swiglu_bwd: a pointer is not aligned to its element size");
     const int mode = swiglu_mode(H * es, aligned(dgu, 16) && aligned(dh, 16) && aligned(gu, 16));
-    drop_stale_error();
     hipError_t e =
         launch_swiglu_bwd(dtype, mode, swiglu_unroll(1, 4), xcd_group_or(kXcdGroupStreaming), dgu, dh, gu, (long)M, (long)H, (hipStream_t)stream);
     if (e != hipSuccess) return fail_hip("mg_swiglu_bwd: launch", e);

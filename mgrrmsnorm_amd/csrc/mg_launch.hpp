@@ -4,7 +4,30 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 namespace mg {
+
+// Kernel launch whose return value is this launch's own status.  hipLaunchKernel reports it
+// directly, so nothing has to be read from the thread's last-error slot, which other users of
+// the HIP runtime in the process (torch) share: an error they left there stays where it is.
+// When our launch fails, the runtime has put that error into the slot as well; it is ours and
+// is taken out again, so that it does not surface in somebody else's next check.
+template <typename... P, size_t... I>
+hipError_t launch_unpacked(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t s,
+                           std::tuple<P...>& vals, std::index_sequence<I...>) {
+    void* ptrs[] = {static_cast<void*>(&std::get<I>(vals))...};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds_bytes, s);
+    if (e != hipSuccess) (void)hipGetLastError();
+    return e;
+}
+template <typename... P, typename... A>
+hipError_t launch(void (*kernel)(P...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t s, A... args) {
+    static_assert(sizeof...(P) == sizeof...(A), "one argument per kernel parameter");
+    std::tuple<P...> vals{static_cast<P>(args)...};
+    return launch_unpacked(kernel, grid, block, lds_bytes, s, vals, std::index_sequence_for<P...>{});
+}
 
 // How a row is spread over threads in the register-resident RMSNorm kernels.
 struct RowCfg {

@@ -25,10 +25,9 @@ hipError_t run(const BwdArgs& a, hipStream_t s) {
     if constexpr (bwd_cfg_ok((int)sizeof(elem_t), TPR, ITEMS, BLOCK)) {
         auto kernel = a.prefetch ? rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK, true>
                                  : rmsnorm_bwd_rows<elem_t, kVec, TPR, ITEMS, BLOCK, false>;
-        kernel<<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
-                (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
+        return launch(kernel, dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s,
+            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w,
                 a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);
-        return hipGetLastError();
     } else {
         return hipErrorInvalidValue;
     }
@@ -51,10 +50,9 @@ hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
             if (e != hipSuccess) return e;
             if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
         }
-        kernel<<<dim3((unsigned)a.num_partials), dim3(1024), kLdsBytes, s>>>(
+        return launch(kernel, dim3((unsigned)a.num_partials), dim3(1024), kLdsBytes, s,
             (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
             a.rows, a.cols, 1.0f / (float)a.cols, a.xcd_group);
-        return hipGetLastError();
     } else {
         return hipErrorInvalidValue;
     }
@@ -63,10 +61,9 @@ hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
 template <int TPR, int ITEMS, int DEPTH>
 hipError_t run_ring(const BwdArgs& a, hipStream_t s) {
     constexpr int BLOCK = TPR > 512 ? TPR : 512;
-    rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH><<<dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s>>>(
-        (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+    return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH>, dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s,
+            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
         a.rows, a.cols, 1.0f / (float)a.cols);
-    return hipGetLastError();
 }
 
 template <int TPR, int ITEMS>
@@ -101,18 +98,16 @@ hipError_t by_items(int items, const BwdArgs& a, hipStream_t s) {
 
 template <int TPR, int ITEMS, bool RAGGED>
 hipError_t run_narrow(const BwdArgs& a, hipStream_t s) {
-    rmsnorm_bwd_narrow<elem_t, TPR, ITEMS, RAGGED><<<dim3((unsigned)a.num_partials), dim3(512), 0, s>>>(
-        (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+    return launch(rmsnorm_bwd_narrow<elem_t, TPR, ITEMS, RAGGED>, dim3((unsigned)a.num_partials), dim3(512), 0, s,
+            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
         a.rows, a.cols, 1.0f / (float)a.cols);
-    return hipGetLastError();
 }
 
 template <int TPR, int G, bool RAGGED, int POL>
 hipError_t run_groups(const BwdArgs& a, hipStream_t s) {
-    rmsnorm_bwd_groups<elem_t, TPR, G, RAGGED, POL><<<dim3((unsigned)a.num_partials), dim3(512), 0, s>>>(
-        (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
+    return launch(rmsnorm_bwd_groups<elem_t, TPR, G, RAGGED, POL>, dim3((unsigned)a.num_partials), dim3(512), 0, s,
+            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
         a.rows, a.cols, 1.0f / (float)a.cols);
-    return hipGetLastError();
 }
 
 // ragged rows (pitch not a multiple of 16 bytes) take the default cache policy, as in the
@@ -167,27 +162,21 @@ hipError_t by_tpr(int tpr, int items, const BwdArgs& a, hipStream_t s) {
 template <>
 hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const BwdArgs& a, hipStream_t s) {
     if (generic) {
-        rmsnorm_bwd_dx_generic<elem_t><<<dim3((unsigned)a.rows), dim3(256), 0, s>>>(
+        hipError_t e = launch(rmsnorm_bwd_dx_generic<elem_t>, dim3((unsigned)a.rows), dim3(256), 0, s,
             (elem_t*)a.dx, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows,
             a.cols, 1.0f / (float)a.cols);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        rmsnorm_bwd_dw_generic<elem_t>
-            <<<dim3((unsigned)((a.cols + 255) / 256), (unsigned)a.num_partials), dim3(256), 0, s>>>(
-                a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
-        return hipGetLastError();
+        return launch(rmsnorm_bwd_dw_generic<elem_t>, dim3((unsigned)((a.cols + 255) / 256), (unsigned)a.num_partials), dim3(256), 0, s,
+            a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
     }
     if (cfg.family == kFamilyStreaming) {
-        rmsnorm_bwd_dx_wide<elem_t><<<dim3((unsigned)a.rows), dim3(kWideBlock), 0, s>>>(
+        hipError_t e = launch(rmsnorm_bwd_dx_wide<elem_t>, dim3((unsigned)a.rows), dim3(kWideBlock), 0, s,
             (elem_t*)a.dx, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows, a.cols,
             1.0f / (float)a.cols);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
         const long nvec = ((long)a.cols * (long)sizeof(elem_t) + kVec - 1) / kVec;
-        rmsnorm_bwd_dw_wide<elem_t>
-            <<<dim3((unsigned)((nvec + 255) / 256), (unsigned)a.num_partials), dim3(256), 0, s>>>(
-                a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
-        return hipGetLastError();
+        return launch(rmsnorm_bwd_dw_wide<elem_t>, dim3((unsigned)((nvec + 255) / 256), (unsigned)a.num_partials), dim3(256), 0, s,
+            a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, a.inv_rms, a.rows, a.cols);
     }
     if (cfg.vec != kVec) return hipErrorInvalidValue;
     if (cfg.family == kFamilyLdsSums) {

@@ -23,10 +23,9 @@ hipError_t run(const FwdArgs& a, hipStream_t s) {
     constexpr int BLOCK = TPR > 256 ? TPR : 256;
     constexpr int RPB = BLOCK / TPR;
     const long grid = (a.rows + RPB - 1) / RPB;
-    rmsnorm_fwd_rows<elem_t, VEC, TPR, ITEMS><<<dim3((unsigned)grid), dim3(BLOCK), 0, s>>>(
-        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+    return launch(rmsnorm_fwd_rows<elem_t, VEC, TPR, ITEMS>, dim3((unsigned)grid), dim3(BLOCK), 0, s,
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
         1.0f / (float)a.cols, a.xcd_group);
-    return hipGetLastError();
 }
 
 template <int VEC, int TPR>
@@ -47,20 +46,18 @@ template <int TPR, int ITEMS, bool RAGGED>
 hipError_t run_narrow(const FwdArgs& a, hipStream_t s) {
     constexpr int RPB = 256 / TPR;
     const long grid = (a.rows + RPB - 1) / RPB;
-    rmsnorm_fwd_narrow<elem_t, TPR, ITEMS, RAGGED><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
-        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+    return launch(rmsnorm_fwd_narrow<elem_t, TPR, ITEMS, RAGGED>, dim3((unsigned)grid), dim3(256), 0, s,
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
         1.0f / (float)a.cols, a.xcd_group);
-    return hipGetLastError();
 }
 
 template <int TPR, int G, bool RAGGED, int POL>
 hipError_t run_groups(const FwdArgs& a, hipStream_t s) {
     constexpr int RPB = 4 * G * (kWave / TPR);
     const long grid = (a.rows + RPB - 1) / RPB;
-    rmsnorm_fwd_groups<elem_t, TPR, G, RAGGED, POL><<<dim3((unsigned)grid), dim3(256), 0, s>>>(
-        (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+    return launch(rmsnorm_fwd_groups<elem_t, TPR, G, RAGGED, POL>, dim3((unsigned)grid), dim3(256), 0, s,
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
         1.0f / (float)a.cols, a.xcd_group);
-    return hipGetLastError();
 }
 
 // ragged rows (pitch not a multiple of 16 bytes) take the default cache policy, as in the
@@ -116,16 +113,14 @@ hipError_t by_tpr(int tpr, int items, const FwdArgs& a, hipStream_t s) {
 template <>
 hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const FwdArgs& a, hipStream_t s) {
     if (generic) {
-        rmsnorm_fwd_generic<elem_t><<<dim3((unsigned)a.rows), dim3(256), 0, s>>>(
+        return launch(rmsnorm_fwd_generic<elem_t>, dim3((unsigned)a.rows), dim3(256), 0, s,
             (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
             1.0f / (float)a.cols);
-        return hipGetLastError();
     }
     if (cfg.family == kFamilyStreaming) {
-        rmsnorm_fwd_wide<elem_t><<<dim3((unsigned)a.rows), dim3(kWideBlock), 0, s>>>(
+        return launch(rmsnorm_fwd_wide<elem_t>, dim3((unsigned)a.rows), dim3(kWideBlock), 0, s,
             (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
             1.0f / (float)a.cols);
-        return hipGetLastError();
     }
     if (cfg.family == kFamilyGroups) {
         if (!groups_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items)) return hipErrorInvalidValue;

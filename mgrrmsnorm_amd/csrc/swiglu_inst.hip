@@ -104,9 +104,8 @@ hipError_t fwd_vec(int xg, void* h, const void* gu, long M, long H, hipStream_t 
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * nvr);
         const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
-        swiglu_fwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_fwd_vec<T, UNROLL>, dim3(grid), dim3(256), 0, s,
             (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd, xg);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -121,9 +120,8 @@ hipError_t bwd_vec(int xg, void* dgu, const void* dh, const void* gu, long M, lo
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * nvr);
         const unsigned grid = (unsigned)((total + 256u * UNROLL - 1) / (256u * UNROLL));
-        swiglu_bwd_vec<T, UNROLL><<<dim3(grid), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_bwd_vec<T, UNROLL>, dim3(grid), dim3(256), 0, s,
             (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd, xg);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -146,9 +144,8 @@ hipError_t fwd_ragged(int xg, void* h, const void* gu, long M, long H, hipStream
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * nvr);
-        swiglu_fwd_ragged<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_fwd_ragged<T>, dim3((total + 255u) / 256u), dim3(256), 0, s,
             (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, (uint32_t)m, total, (uint32_t)half_bytes, fd, xg);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -163,10 +160,9 @@ hipError_t bwd_ragged(int xg, void* dgu, const void* dh, const void* gu, long M,
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * nvr);
-        swiglu_bwd_ragged<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_bwd_ragged<T>, dim3((total + 255u) / 256u), dim3(256), 0, s,
             (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, (uint32_t)m, total,
             (uint32_t)half_bytes, fd, xg);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -179,9 +175,8 @@ hipError_t fwd_gen(void* h, const void* gu, long M, long H, hipStream_t s) {
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * H);
-        swiglu_fwd_generic<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_fwd_generic<T>, dim3((total + 255u) / 256u), dim3(256), 0, s,
             (T*)h + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -194,9 +189,8 @@ hipError_t bwd_gen(void* dgu, const void* dh, const void* gu, long M, long H, hi
     for (long r0 = 0; r0 < M; r0 += rows_per_launch) {
         const long m = (M - r0) < rows_per_launch ? (M - r0) : rows_per_launch;
         const uint32_t total = (uint32_t)(m * H);
-        swiglu_bwd_generic<T><<<dim3((total + 255u) / 256u), dim3(256), 0, s>>>(
+        hipError_t e = launch(swiglu_bwd_generic<T>, dim3((total + 255u) / 256u), dim3(256), 0, s,
             (T*)dgu + r0 * 2 * H, (const T*)dh + r0 * H, (const T*)gu + r0 * 2 * H, total, fd);
-        hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
@@ -257,39 +251,36 @@ hipError_t launch_swiglu_bwd(int dtype, int mode, int unroll, int xg, void* dgu,
 hipError_t launch_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* part, int P, int ld,
                             int cols, hipStream_t s) {
     const dim3 grid((unsigned)((cols + kReduceCols - 1) / kReduceCols)), block(256);
-    if (dw_cast == nullptr || cast_dtype == MG_F32) {
-        rmsnorm_dw_reduce<float><<<grid, block, 0, s>>>(dw_f32, (float*)dw_cast, part, P, ld, cols);
-    } else if (cast_dtype == MG_F16) {
-        rmsnorm_dw_reduce<half_t><<<grid, block, 0, s>>>(dw_f32, (half_t*)dw_cast, part, P, ld, cols);
-    } else if (cast_dtype == MG_BF16) {
-        rmsnorm_dw_reduce<bf16_t><<<grid, block, 0, s>>>(dw_f32, (bf16_t*)dw_cast, part, P, ld, cols);
-    } else {
-        return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
+    if (dw_cast == nullptr || cast_dtype == MG_F32)
+        return launch(rmsnorm_dw_reduce<float>, grid, block, 0, s, dw_f32, (float*)dw_cast, part, P, ld, cols);
+    if (cast_dtype == MG_F16)
+        return launch(rmsnorm_dw_reduce<half_t>, grid, block, 0, s, dw_f32, (half_t*)dw_cast, part, P, ld, cols);
+    if (cast_dtype == MG_BF16)
+        return launch(rmsnorm_dw_reduce<bf16_t>, grid, block, 0, s, dw_f32, (bf16_t*)dw_cast, part, P, ld, cols);
+    return hipErrorInvalidValue;
 }
 
 hipError_t launch_copy(void* dst, const void* src, long bytes, hipStream_t s) {
     const long n = bytes / 16;
     if (n <= 0) return hipSuccess;
-    copy_vec16<<<dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s>>>((u32x4*)dst, (const u32x4*)src, n);
-    return hipGetLastError();
+    return launch(copy_vec16, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (u32x4*)dst, (const u32x4*)src, n);
 }
 
 hipError_t launch_stream_probe(void* dst, const void* a, const void* b, long bytes, int xcd_group, hipStream_t s) {
     const long n = (bytes + 4095) / 4096;
     if (n <= 0) return hipSuccess;
     if (b == nullptr)
-        stream_probe<false><<<dim3((unsigned)n), dim3(256), 0, s>>>((char*)dst, (const char*)a, nullptr, bytes, xcd_group);
-    else
-        stream_probe<true><<<dim3((unsigned)n), dim3(256), 0, s>>>((char*)dst, (const char*)a, (const char*)b, bytes, xcd_group);
-    return hipGetLastError();
+        return launch(stream_probe<false>, dim3((unsigned)n), dim3(256), 0, s, (char*)dst, (const char*)a,
+                      (const char*)nullptr, bytes, xcd_group);
+    return launch(stream_probe<true>, dim3((unsigned)n), dim3(256), 0, s, (char*)dst, (const char*)a, (const char*)b,
+                  bytes, xcd_group);
 }
 
 template <bool TWO_READS>
 hipError_t row_probe_by_shape(unsigned grid, void* dst, const void* a, const void* b, long rows, u32 row_bytes,
                               hipStream_t s) {
-#define MG_ROW_PROBE(B, I) row_probe<TWO_READS, B, I><<<dim3(grid), dim3(B), 0, s>>>((char*)dst, (const char*)a, (const char*)b, rows, row_bytes)
+#define MG_ROW_PROBE(B, I) \
+    return launch(row_probe<TWO_READS, B, I>, dim3(grid), dim3(B), 0, s, (char*)dst, (const char*)a, (const char*)b, rows, row_bytes)
     const u32 nvec = row_bytes / 16u;
     if (nvec <= 256) MG_ROW_PROBE(256, 1);
     else if (nvec <= 512) MG_ROW_PROBE(512, 1);
@@ -297,7 +288,6 @@ hipError_t row_probe_by_shape(unsigned grid, void* dst, const void* a, const voi
     else if (nvec <= 2048) MG_ROW_PROBE(1024, 2);
     else MG_ROW_PROBE(1024, 4);
 #undef MG_ROW_PROBE
-    return hipGetLastError();
 }
 
 hipError_t launch_row_probe(void* dst, const void* a, const void* b, long rows, long row_bytes, long workgroups,
@@ -311,8 +301,7 @@ hipError_t launch_row_probe(void* dst, const void* a, const void* b, long rows, 
 hipError_t launch_fill_zero(float* p, long n, hipStream_t s) {
     if (n <= 0) return hipSuccess;
     const long blocks = (n + 255) / 256;
-    fill_zero_f32<<<dim3((unsigned)(blocks < (1L << 20) ? blocks : (1L << 20))), dim3(256), 0, s>>>(p, n);
-    return hipGetLastError();
+    return launch(fill_zero_f32, dim3((unsigned)(blocks < (1L << 20) ? blocks : (1L << 20))), dim3(256), 0, s, p, n);
 }
 
 }  // namespace mg

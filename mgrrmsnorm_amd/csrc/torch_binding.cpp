@@ -236,6 +236,8 @@ Tensor swiglu(const Tensor& w12_out, int64_t hidden_dim) {
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "torch extension over libmegagemm_hip.so (C ABI version " + std::to_string(MG_ABI_VERSION) + ")";
     m.def("abi_version", [] { return mg_abi_version(); }, "ABI version of the loaded libmegagemm_hip.so");
+    m.def("built_abi_version", [] { return MG_ABI_VERSION; },
+          "MG_ABI_VERSION of the header this extension was compiled against");
     m.def("rmsnorm_forward", &rmsnorm_forward, "RMSNorm forward: [output, inv_rms]", py::arg("input"),
           py::arg("weight"), py::arg("epsilon"));
     m.def("rmsnorm_backward", &rmsnorm_backward, "RMSNorm backward: [grad_input, grad_weight]",

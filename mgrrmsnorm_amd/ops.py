@@ -26,6 +26,18 @@ _binding = None
 _resolved = False
 
 
+def _check_extension_abi(ext) -> None:
+    """The extension must have been compiled against this package's header (its own
+    MG_ABI_VERSION constant) and must have loaded a library of the same version."""
+    built = getattr(ext, "built_abi_version", lambda: None)()
+    if built != _lib.ABI_VERSION:
+        raise RuntimeError(f"{ext.__file__} was compiled against ABI {built}, "
+                           f"this package needs {_lib.ABI_VERSION}; rebuild it")
+    if ext.abi_version() != _lib.ABI_VERSION:
+        raise RuntimeError(f"{ext.__file__} loaded a libmegagemm_hip.so of ABI {ext.abi_version()}, "
+                           f"this package needs {_lib.ABI_VERSION}; rebuild it")
+
+
 def _extension():
     """The compiled extension module, or None when it is not built / not wanted."""
     global _binding, _resolved
@@ -35,9 +47,7 @@ def _extension():
         try:
             from . import _binding as ext
 
-            if ext.abi_version() != _lib.ABI_VERSION:
-                raise RuntimeError(f"{ext.__file__} was built for ABI {ext.abi_version()}, "
-                                   f"this package needs {_lib.ABI_VERSION}; rebuild it")
+            _check_extension_abi(ext)
             _binding = ext
         except ImportError:
             _binding = None      # not built (or the HIP library is missing: ctypes then says so)

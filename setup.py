@@ -16,9 +16,12 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 
-def _compile_library(out_dir=None):
+def _compile_library(out_dir=None, only_if_stale=False):
     from mgrrmsnorm_amd import _build
 
+    if only_if_stale and out_dir is None and _build.is_current():
+        print(f"{_build.LIB_PATH.name} and {_build.BINDING_PATH.name} are newer than their sources: not rebuilt")
+        return
     print(f"building {_build.LIB_PATH.name} for {_build.ARCH} and {_build.BINDING_PATH.name}"
           + (f" into {out_dir}" if out_dir else ""))
     _build.build(out_dir=out_dir)
@@ -39,14 +42,20 @@ class BuildHip(Command):
 
 
 class BuildPyWithHip(build_py):
+    """`pip install .` / `python setup.py build`: compile in the source tree (unless what is
+    there is newer than its sources), then let build_py copy package data, the built files
+    among them."""
+
     def run(self):
-        _compile_library()
+        _compile_library(only_if_stale=True)
         super().run()
 
 
 class DevelopWithHip(develop):
+    """`pip install -e .`: the same compile step; the package then runs from the source tree."""
+
     def run(self):
-        _compile_library()
+        _compile_library(only_if_stale=True)
         super().run()
 
 

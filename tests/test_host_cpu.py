@@ -12,11 +12,39 @@ def test_lazy_exports_and_unknown_attribute():
     import mgrrmsnorm_amd as m
 
     assert m.__version__ == "0.1.0"
-    assert set(m.__all__) == {"RMSNorm", "RMSNormFunction", "MegaGemmTriton", "MegaGemmFunction", "__version__"}
+    # the reference's four names and version; the one addition is the autograd-threading helper
+    assert set(m.__all__) == {"RMSNorm", "RMSNormFunction", "MegaGemmTriton", "MegaGemmFunction", "__version__",
+                              "backward_on_calling_thread"}
     for name in ("RMSNorm", "RMSNormFunction", "MegaGemmTriton", "MegaGemmFunction"):
         assert getattr(m, name).__name__ == name
     with pytest.raises(AttributeError, match="has no attribute 'Nope'"):
         m.Nope
+
+
+def test_backward_on_calling_thread_wraps_torchs_switch():
+    import threading
+
+    import megagemm
+
+    seen = []
+
+    class Probe(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            return x * 2
+
+        @staticmethod
+        def backward(ctx, g):
+            seen.append(threading.get_ident())
+            return g * 2
+
+    assert torch.autograd.is_multithreading_enabled()
+    with megagemm.backward_on_calling_thread():
+        assert not torch.autograd.is_multithreading_enabled()
+        x = torch.ones(4, requires_grad=True)
+        Probe.apply(x).sum().backward()
+    assert torch.autograd.is_multithreading_enabled()
+    assert seen == [threading.get_ident()] and torch.equal(x.grad, torch.full((4,), 2.0))
 
 
 def test_megagemm_alias_package():

@@ -282,6 +282,53 @@ def test_full_size_by_row_replication(dtype, rows, cols):
     U.assert_dw(dw, dw_ref * reps, "dW = reps x block dW")
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16", "fp32"])
+def test_one_column_rows_are_all_cancellation(dtype):
+    """With a single column dx = s*dy*w - x*s^3*(dy*w*x) = s*dy*w*eps/(x^2+eps): the difference of
+    two terms that agree to about eps/x^2 of their size, in every element.  No fp32 evaluation of
+    the reference's formula resolves that to 1 ulp of the result (its own literal restatement
+    misses at most elements as well), so this shape is held to the error bound of the subtraction,
+    4 * 2^-24 * (|term 1| + |term 2|), in every element, and the counts are printed: that is the
+    one place where the share of elements passing through the floor is not capped."""
+    rows, cols = 629, 1
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=9)
+    y_ref, s_ref, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    y, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    U.assert_matches(y, y_ref, dtype, "y, one column")
+    dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    n_floor = U.assert_matches(dx, dx_ref, dtype, "dx, one column", floor=floor, every_element_cancels=True)
+    U.assert_dw(dw, dw_ref)
+    # the same count for the reference's own arithmetic in fp32, rounded once
+    ref32 = torch.from_numpy(floor.ref32.astype(np.float32)).to(U.DTYPES[dtype])
+    n_ref = U.assert_matches(ref32, dx_ref, dtype, "dx, one column, reference fp32 arithmetic", floor=floor.bound,
+                             every_element_cancels=True)
+    print(f"one column [{dtype}]: {n_floor} of {rows} elements of dx beyond 1 ulp / 1e-5 (within the floor); "
+          f"the reference's fp32 arithmetic: {n_ref}")
+    assert n_floor > 0 and n_ref > 0, "this shape is expected to need the floor on both sides"
+
+
+@pytest.mark.parametrize("rows,cols,outliers", [(4096, 4096, False), (1024, 8192, False), (2048, 768, True),
+                                                (2048, 2048, True), (1024, 4100, True), (1024, 5120, True),
+                                                (512, 16384, True)])
+def test_fp32_dx_beyond_1e5_before_the_floor_at_benchmark_widths(rows, cols, outliers):
+    """The benchmark configurations' widths and input recipes in fp32: how many elements of dx
+    miss the 1e-5 relative bar before the cancellation floor is applied, next to the count for
+    the literal fp32 restatement of the reference's arithmetic.  The kernel may need the floor at
+    no more elements than 5e-3 of the tensor plus that count."""
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "fp32", seed=42, outliers=outliers)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, "fp32")
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, "fp32")
+    dx, dw, _, _ = U.rmsnorm_bwd(dyd, xd, wd, s, "fp32")
+    n_floor = U.assert_matches(dx, dx_ref, "fp32", f"dx, {rows}x{cols} fp32", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    rel = np.abs(floor.ref32.astype(np.float64) - dx_ref) > 1e-5 * np.abs(dx_ref) + 1e-37
+    print(f"{rows}x{cols} fp32{' with outliers' if outliers else ''}: {n_floor} of {rows * cols} elements of dx "
+          f"({n_floor / (rows * cols):.2e}) beyond 1e-5 relative before the floor; the reference's fp32 arithmetic: "
+          f"{int(rel.sum())} ({rel.mean():.2e})")
+
+
 @pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("bf16", 16384, 8192), ("bf16", 65536, 768),
                                              ("fp32", 4096, 4096), ("bf16", 1048576, 64)])
 def test_power_of_two_scaling_is_exact(dtype, rows, cols):

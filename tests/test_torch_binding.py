@@ -23,7 +23,8 @@ def test_module_surface_and_host_side_checks(binding):
     for name in ("rmsnorm_forward", "rmsnorm_backward", "rmsnorm_backward_f32", "swiglu_forward", "swiglu_backward",
                  "rmsnorm", "swiglu"):
         assert callable(getattr(binding, name)), name
-    assert binding.abi_version() == _lib.ABI_VERSION
+    assert binding.abi_version() == _lib.ABI_VERSION          # the library it loaded
+    assert binding.built_abi_version() == _lib.ABI_VERSION    # the header it was compiled against
     assert ops.backend() == "extension"      # the package uses it as soon as it is built
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         binding.rmsnorm_forward(torch.ones(2, 8), torch.ones(8), 1e-6)
@@ -31,6 +32,27 @@ def test_module_surface_and_host_side_checks(binding):
         binding.swiglu_forward(torch.ones(2, 8), 4)
     with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
         binding.rmsnorm(torch.ones(2, 8), torch.ones(8), 1e-6)
+
+
+def test_stale_extension_is_refused():
+    """An extension compiled against another version of the header, or one without the
+    compile-time constant at all (built before it existed), must not be used."""
+    import types
+
+    from mgrrmsnorm_amd import _lib, ops
+
+    v = _lib.ABI_VERSION
+    ok = types.SimpleNamespace(__file__="x.so", abi_version=lambda: v, built_abi_version=lambda: v)
+    ops._check_extension_abi(ok)
+    old_header = types.SimpleNamespace(__file__="x.so", abi_version=lambda: v, built_abi_version=lambda: v - 1)
+    with pytest.raises(RuntimeError, match=f"compiled against ABI {v - 1}"):
+        ops._check_extension_abi(old_header)
+    no_constant = types.SimpleNamespace(__file__="x.so", abi_version=lambda: v)
+    with pytest.raises(RuntimeError, match="compiled against ABI None"):
+        ops._check_extension_abi(no_constant)
+    old_library = types.SimpleNamespace(__file__="x.so", abi_version=lambda: v + 1, built_abi_version=lambda: v)
+    with pytest.raises(RuntimeError, match=f"loaded a libmegagemm_hip.so of ABI {v + 1}"):
+        ops._check_extension_abi(old_library)
 
 
 @pytest.mark.gpu
