@@ -127,7 +127,10 @@ int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const flo
  * as dw_f32 ([cols] fp32) and/or dw_cast ([cols] of `dtype`); at least one of the two -- but
  * keeps the dW partials in a device array of MG_NOALLOC_SCRATCH_BYTES that belongs to the
  * library (one copy per GPU the library runs on, held until the process ends) instead of a
- * workspace of the caller's.  It calls no allocating routine.  The number of partial rows is
+ * workspace of the caller's.  That array is part of the library's code object, so its cost --
+ * 16 MiB of device memory on every GPU on which the process uses the library -- is paid by every
+ * user of the library from the moment the code object is loaded, whether or not this entry
+ * point is ever called.  It calls no allocating routine.  The number of partial rows is
  * the one mg_rmsnorm_bwd_workspace reports, capped at MG_NOALLOC_SCRATCH_BYTES / (4 * ld);
  * results are bit-identical to the two-call sequence with that number of partial rows.
  * cols above MG_NOALLOC_MAX_COLS is rejected with MG_ERR_UNSUPPORTED.

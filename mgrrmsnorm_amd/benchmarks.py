@@ -2,13 +2,17 @@
 this package, wall-clock per call with a device synchronisation on both sides.
 
     python -m mgrrmsnorm_amd.benchmarks swiglu     # benchmark_swiglu.py:61-181 (block forward, 3 configs)
-    python -m mgrrmsnorm_amd.benchmarks rmsnorm    # colab_test.py:143-184 / README.md:28-35 (fp16 forward)
+    python -m mgrrmsnorm_amd.benchmarks rmsnorm    # colab_test.py:143-184 / README.md:28-35: forward and
+                                                   # forward+backward, fp16 and bf16
     python -m mgrrmsnorm_amd.benchmarks all
 
 Method as in the reference (benchmark_swiglu.py:16-37): 10 warm-up calls, then 100 calls each
 bracketed by torch.cuda.synchronize() and time.perf_counter(); mean and standard deviation
-in milliseconds, speed-up of this package over PyTorch, peak device memory.  For kernel-level
-bandwidth figures use bench.py at the repository root instead.
+in milliseconds, speed-up of this package over PyTorch, peak device memory.  A call of 13-35 us
+of GPU work timed that way is mostly the latency of one launch and one synchronisation, the
+same for every implementation, so the RMSNorm tables carry a second column: GPU time per call,
+from device events around the same calls issued back to back.  For kernel-level bandwidth
+figures use bench.py at the repository root instead.
 """
 from __future__ import annotations
 
@@ -55,14 +59,40 @@ class UnfusedSwiGLU(torch.nn.Module):
         return self.w3(F.silu(self.w1(x)) * self.w2(x))
 
 
+def gpu_time_per_call(fn, warmup: int = 10, iterations: int = 100):
+    """GPU time of fn() in milliseconds: device events around `iterations` calls issued back to
+    back (no synchronisation in between), best of three."""
+    for _ in range(warmup):
+        fn()
+    best = None
+    for _ in range(3):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(iterations):
+            fn()
+        b.record()
+        b.synchronize()
+        t = a.elapsed_time(b) / iterations
+        best = t if best is None else min(best, t)
+    return best
+
+
 def _report(title, rows):
-    print(f"\n{'=' * 64}\n{title}\n{'=' * 64}")
-    print(f"{'Implementation':<26}{'Time (ms)':<22}{'Speedup':>10}")
-    print("-" * 64)
+    """rows: (name, mean ms, std ms[, GPU ms per call])."""
+    with_gpu = len(rows[0]) > 3
+    width = 84 if with_gpu else 64
+    print(f"\n{'=' * width}\n{title}\n{'=' * width}")
+    print(f"{'Implementation':<26}{'Time (ms)':<22}{'Speedup':>10}" + (f"{'GPU time (ms)':>16}{'':>4}" if with_gpu else ""))
+    print("-" * width)
     base = rows[0][1]
-    for name, mean, std in rows:
-        print(f"{name:<26}{mean:>8.3f} +/- {std:<8.3f}{base / mean:>12.2f}x")
-    print("=" * 64)
+    for row in rows:
+        name, mean, std = row[:3]
+        line = f"{name:<26}{mean:>8.3f} +/- {std:<8.3f}{base / mean:>12.2f}x"
+        if with_gpu:
+            line += f"{row[3]:>14.4f} {rows[0][3] / row[3]:>5.2f}x"
+        print(line)
+    print("=" * width)
 
 
 def bench_swiglu(dtype=torch.float16, configs=None, warmup: int = 10, iterations: int = 100):
@@ -92,31 +122,50 @@ def bench_swiglu(dtype=torch.float16, configs=None, warmup: int = 10, iterations
     return results
 
 
-def bench_rmsnorm(dtype=torch.float16, configs=None, warmup: int = 10, iterations: int = 100):
-    """Forward, PyTorch formula and torch.nn.RMSNorm against this package; returns
-    {(batch, seq, hidden): {"formula_ms", "native_ms", "hip_ms": (mean, std), "max_diff": float}}."""
+def bench_rmsnorm(dtype=torch.float16, configs=None, warmup: int = 10, iterations: int = 100, backward: bool = False):
+    """Forward (or forward + backward), PyTorch formula and torch.nn.RMSNorm against this package;
+    returns {(batch, seq, hidden): {"formula_ms", "native_ms", "hip_ms": (mean, std), "formula_gpu_ms",
+    "native_gpu_ms", "hip_gpu_ms": float, "max_diff": float}}."""
     results = {}
     for batch, seq, hidden in (RMSNORM_CONFIGS if configs is None else configs):
-        x = torch.randn(batch, seq, hidden, device="cuda", dtype=dtype)
+        x = torch.randn(batch, seq, hidden, device="cuda", dtype=dtype, requires_grad=backward)
+        dy = torch.randn(batch, seq, hidden, device="cuda", dtype=dtype)
         ours = RMSNorm(hidden, 1e-6).cuda().to(dtype)
         native = torch.nn.RMSNorm(hidden, eps=1e-6).cuda().to(dtype)
-        w = ours.weight.detach()
+        w = ours.weight if backward else ours.weight.detach()
 
         def formula():                               # colab_test.py:176
             return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
 
+        def run(f):
+            if not backward:
+                return lambda: f()
+
+            def step():
+                x.grad = None
+                ours.weight.grad = None
+                native.weight.grad = None
+                f().backward(dy)
+            return step
+
+        calls = [("PyTorch formula", run(formula)), ("torch.nn.RMSNorm", run(lambda: native(x))),
+                 ("mgrrmsnorm_amd (HIP)", run(lambda: ours(x)))]
+        import contextlib
+
+        with (contextlib.nullcontext() if backward else torch.no_grad()):
+            wall = [time_calls(f, warmup, iterations) for _, f in calls]
+            gpu = [gpu_time_per_call(f, warmup, iterations) for _, f in calls]
         with torch.no_grad():
-            t_formula = time_calls(formula, warmup, iterations)
-            t_native = time_calls(lambda: native(x), warmup, iterations)
-            t_ours = time_calls(lambda: ours(x), warmup, iterations)
             diff = (formula().float() - ours(x).float()).abs().max().item()
-        _report(f"RMSNorm forward  batch={batch} seq={seq} hidden={hidden} {dtype}",
-                [("PyTorch formula", *t_formula), ("torch.nn.RMSNorm", *t_native), ("mgrrmsnorm_amd (HIP)", *t_ours)])
+        what = "forward + backward" if backward else "forward"
+        _report(f"RMSNorm {what}  batch={batch} seq={seq} hidden={hidden} {dtype}",
+                [(name, *wall[i], gpu[i]) for i, (name, _) in enumerate(calls)])
         tokens = batch * seq
-        print(f"tokens per second: PyTorch formula {tokens / t_formula[0] * 1e3:,.0f}, "
-              f"this package {tokens / t_ours[0] * 1e3:,.0f}")
+        print(f"tokens per second: PyTorch formula {tokens / wall[0][0] * 1e3:,.0f}, "
+              f"this package {tokens / wall[2][0] * 1e3:,.0f}")
         print(f"max |difference| vs the formula = {diff:.6f}")
-        results[(batch, seq, hidden)] = {"formula_ms": t_formula, "native_ms": t_native, "hip_ms": t_ours,
+        results[(batch, seq, hidden)] = {"formula_ms": wall[0], "native_ms": wall[1], "hip_ms": wall[2],
+                                         "formula_gpu_ms": gpu[0], "native_gpu_ms": gpu[1], "hip_gpu_ms": gpu[2],
                                          "max_diff": diff}
     return results
 
@@ -130,7 +179,9 @@ def main(argv=None):
         raise SystemExit("no GPU visible")
     print(f"GPU: {torch.cuda.get_device_name()}   PyTorch: {torch.__version__}")
     if what in ("rmsnorm", "all"):
-        bench_rmsnorm()
+        for dtype in (torch.float16, torch.bfloat16):
+            bench_rmsnorm(dtype=dtype)
+            bench_rmsnorm(dtype=dtype, backward=True)
     if what in ("swiglu", "all"):
         bench_swiglu()
 

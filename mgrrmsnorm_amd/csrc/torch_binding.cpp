@@ -214,10 +214,26 @@ struct SwigluNode : public torch::autograd::Function<SwigluNode> {
 Tensor rmsnorm(const Tensor& input, const Tensor& weight, double epsilon) {
     if (torch::GradMode::is_enabled() && (input.requires_grad() || weight.requires_grad()))
         return RMSNormNode::apply(input, weight, epsilon);
-    // nothing to differentiate: same kernel, no node and no saved tensors
+    // nothing to differentiate: same kernel, no node, no saved tensors and no per-row scale
+    // (the C ABI takes a null inv_rms); the output keeps the input's shape, so no views either
     TORCH_CHECK(input.dim() >= 1, "RMSNorm needs at least one dimension");
-    const auto shape = input.sizes();
-    return rmsnorm_forward(input.contiguous().view({-1, shape.back()}), weight.contiguous(), epsilon)[0].view(shape);
+    TORCH_CHECK(input.is_cuda(), "input must be a CUDA tensor");
+    TORCH_CHECK(weight.is_cuda(), "weight must be a CUDA tensor");
+    const Tensor x = input.contiguous(), w = weight.contiguous();   // themselves when they already are
+    const int64_t cols = x.size(-1);
+    TORCH_CHECK(cols >= 1, "hidden size must be >= 1");
+    TORCH_CHECK(w.dim() == 1 && w.size(0) == cols, "Weight size must match hidden size");
+    TORCH_CHECK(w.scalar_type() == x.scalar_type(), "weight dtype (", w.scalar_type(), ") must equal input dtype (",
+                x.scalar_type(), "); cast the module, e.g. model.half() or model.to(torch.bfloat16)");
+    TORCH_CHECK(w.device() == x.device(), "input and weight must be on the same device");
+    const int code = dtype_code(x.scalar_type());
+    const int64_t rows = x.numel() / cols;
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+    auto output = torch::empty_like(x);
+    const int rc = mg_rmsnorm_fwd(output.data_ptr(), nullptr, x.data_ptr(), w.data_ptr(), rows, cols, (float)epsilon,
+                                  code, current_stream());
+    TORCH_CHECK(rc == MG_OK, "RMSNorm forward failed (code ", rc, "): ", mg_last_error());
+    return output;
 }
 
 // silu(gate) * up on a fused [..., 2*hidden_dim] tensor, differentiable.

@@ -33,17 +33,21 @@ def test_swiglu_block_benchmark_default_config_list():
 
 # the formula evaluated by torch in the storage type is itself off by up to an ulp of the
 # output (2^-10 relative in fp16, 2^-7 in bf16; |y| reaches about 4 here)
+@pytest.mark.parametrize("backward", [False, True])
 @pytest.mark.parametrize("dtype,tol", [(torch.float16, 1e-2), (torch.bfloat16, 6.5e-2)])
-def test_rmsnorm_benchmark(dtype, tol, capsys):
+def test_rmsnorm_benchmark(dtype, tol, backward, capsys):
     from mgrrmsnorm_amd import benchmarks
 
     cfg = (4, 32, 1024)
-    res = benchmarks.bench_rmsnorm(dtype=dtype, configs=[cfg], warmup=2, iterations=5)
+    res = benchmarks.bench_rmsnorm(dtype=dtype, configs=[cfg], warmup=2, iterations=5, backward=backward)
     r = res[cfg]
-    assert set(r) == {"formula_ms", "native_ms", "hip_ms", "max_diff"}
+    assert set(r) == {"formula_ms", "native_ms", "hip_ms", "formula_gpu_ms", "native_gpu_ms", "hip_gpu_ms", "max_diff"}
     assert all(r[k][0] > 0 for k in ("formula_ms", "native_ms", "hip_ms"))
+    assert all(r[k] > 0 for k in ("formula_gpu_ms", "native_gpu_ms", "hip_gpu_ms"))
     assert r["max_diff"] < tol
-    assert "tokens per second" in capsys.readouterr().out
+    out = capsys.readouterr().out
+    assert "tokens per second" in out and "GPU time (ms)" in out
+    assert ("forward + backward" in out) == backward
 
 
 def test_time_calls_statistics():
