@@ -538,6 +538,79 @@ def cpu_baseline(wl, budget_s=12.0):
             "sample": f"{sample}; median of {len(times)} runs = {med * 1e3:.2f} ms; host has {os.cpu_count()} logical CPUs"}
 
 
+# ------------------------------------------------------------------------------ timeline
+
+def timeline(wl, lib, launches=40):
+    """Where a launch of backward pass 1 spends its time, from the time stamps of
+    mg_rmsnorm_bwd_timeline (10 ns clock, one record per workgroup): when workgroups start,
+    when their sweeps over the row slots end, when they finish, on which die they ran.
+    Averages over `launches` launches (buffers rotating), all in microseconds, plus what a
+    launch would take if the last sweeps of every workgroup were handed out dynamically
+    instead (a list-scheduling replay of the measured per-workgroup speeds)."""
+    import heapq
+    import statistics as st
+
+    W = 32
+    rec = torch.zeros((wl.P, W), dtype=torch.int64, device="cuda")
+    runs = []
+    for i in range(launches + 4):
+        s = wl.sets[i % wl.nsets]
+        rec.zero_()
+        rc = lib.mg_rmsnorm_bwd_timeline(s["dx"].data_ptr(), wl.partial.data_ptr(), s["dy"].data_ptr(), s["x"].data_ptr(),
+                                         wl.w.data_ptr(), s["inv_rms"].data_ptr(), wl.rows, wl.cols, CODE[wl.dtype],
+                                         wl.P, wl.ld, rec.data_ptr(), stream_ptr())
+        if rc != 0:
+            raise RuntimeError(lib.mg_last_error().decode())
+        torch.cuda.synchronize()
+        if i >= 4:
+            runs.append(rec.cpu().numpy().copy())
+    n_it = int((runs[0][0, 1:25] > 0).sum())
+    us = lambda ticks: ticks * 0.01
+    out = {"workgroups": wl.P, "sweeps_per_workgroup": n_it, "launches": launches}
+    first, med_end, last_end, start_spread, sweep = [], [], [], [], []
+    per_wg = [[] for _ in range(wl.P)]
+    what_if = {}
+    for r in runs:
+        t0 = r[:, 0].min()
+        start, its, loop_end, end = r[:, 0] - t0, r[:, 1:1 + n_it] - t0, r[:, W - 3] - t0, r[:, W - 2] - t0
+        start_spread.append(us(start.max()))
+        first.append(us(float(sorted(its[:, 0])[wl.P // 2])))
+        med_end.append(us(float(sorted(end)[wl.P // 2])))
+        last_end.append(us(float(end.max())))
+        sweep.append(us(float(((its[:, -1] - its[:, 0]) / max(n_it - 1, 1)).mean())))
+        for g in range(wl.P):
+            per_wg[g].append(us(float(end[g])))
+        # replay: the first K sweeps as measured, the remaining (n_it - K) * P sweeps handed to whichever
+        # workgroup is free first, each at that workgroup's own mean sweep time plus `flush` for the partial
+        # row a dynamically assigned unit would have to write (16 KiB) -- what dynamic scheduling could gain
+        for K in (n_it, n_it - 1, n_it - 2, n_it // 2):
+            for flush in (0.0, 0.2, 0.4):
+                per = us((its[:, -1] - start) / n_it)
+                heap = [(us(float(its[g, K - 1])) if K > 0 else us(float(start[g])), g) for g in range(wl.P)]
+                heapq.heapify(heap)
+                fin = [h[0] for h in sorted(heap, key=lambda h: h[1])]
+                for _ in range((n_it - K) * wl.P):
+                    t, g = heapq.heappop(heap)
+                    t += float(per[g]) + flush
+                    fin[g] = t
+                    heapq.heappush(heap, (t, g))
+                tail = us(float((end - its[:, -1]).mean()))
+                what_if.setdefault(f"static_sweeps={K},flush_us={flush}", []).append(max(fin) + tail)
+    mean = lambda v: round(sum(v) / len(v), 2)
+    out.update({"start_spread_us": mean(start_spread), "first_sweep_end_median_us": mean(first),
+                "steady_sweep_us": mean(sweep), "median_workgroup_end_us": mean(med_end),
+                "last_workgroup_end_us": mean(last_end)})
+    means = [sum(v) / len(v) for v in per_wg]
+    out["per_workgroup_mean_end_us"] = {"min": round(min(means), 2), "max": round(max(means), 2),
+                                        "std_of_means": round(st.pstdev(means), 2),
+                                        "mean_std_across_launches": round(sum(st.pstdev(v) for v in per_wg) / wl.P, 2)}
+    xcc = runs[-1][:, W - 1]
+    out["mean_end_us_by_die"] = {int(d): round(sum(m for m, x in zip(means, xcc) if x == d) / max(1, int((xcc == d).sum())), 2)
+                                 for d in sorted(set(int(v) for v in xcc))}
+    out["replay_last_end_us"] = {k: mean(v) for k, v in what_if.items()}
+    return out
+
+
 # ---------------------------------------------------------------------------------- main
 
 def main():
@@ -562,6 +635,10 @@ def main():
     ap.add_argument("--sweep", action="store_true",
                     help="additionally time every configuration of the hidden-size sweep, the large RMSNorm shape "
                          "and the SwiGLU shape (per-kernel and per-step GB/s, table on stderr, 'sweep' in the JSON)")
+    ap.add_argument("--timeline", type=int, default=0, metavar="LAUNCHES",
+                    help="also run backward pass 1 that many times with per-workgroup time stamps "
+                         "(mg_rmsnorm_bwd_timeline; shapes of 4096 two-byte columns) and report where a launch spends "
+                         "its time ('timeline' in the JSON)")
     ap.add_argument("--calibrate-copies", type=int, default=0,
                     help="also launch this many plain copies of one activation tensor (mg_copy_bytes), so that a "
                          "counter profile of this run holds a kernel of known HBM traffic, and as many streaming "
@@ -664,6 +741,8 @@ def main():
         log(f"[bench] ceiling on the same tensors: {section('ceiling', lambda: ceiling(wl))}")
         if isinstance(wl, RmsNormWorkload) and (args.surface == "module" or not args.no_configs):
             log(f"[bench] nn.Module surface: {section('module', lambda: time_module_surface(wl.rows, wl.cols, wl.dtype))}")
+        if args.timeline > 0:
+            log(f"[bench] timeline of backward pass 1: {section('timeline', lambda: timeline(wl, lib, args.timeline))}")
         if not args.no_cpu_baseline:
             log(f"[bench] cpu baseline: {section('cpu_baseline', lambda: cpu_baseline(wl))}")
         del wl

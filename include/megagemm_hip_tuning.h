@@ -66,6 +66,26 @@ int mg_row_probe(void* dst, const void* a, const void* b, int64_t rows, int64_t 
                  int64_t workgroups, void* stream);
 
 /*
+ * mg_rmsnorm_bwd with a clock: the same launch (same results, same arguments), from a build of
+ * the kernel in which thread 0 of every workgroup writes time stamps of the GPU's constant
+ * 100 MHz clock (10 ns units, comparable across workgroups) to records[num_partials]
+ * [MG_TIMELINE_WORDS]: word 0 = start of the workgroup, word 1 + i = end of its i-th sweep over
+ * its row slots (the first MG_TIMELINE_ITERATIONS of them; 0 where there was none), word
+ * MG_TIMELINE_WORDS - 3 = end of the row loop, MG_TIMELINE_WORDS - 2 = end of the workgroup (its
+ * partial row written), MG_TIMELINE_WORDS - 1 = the die (XCC) it ran on.  It shows where a launch
+ * spends its time: how long the first rows take to arrive, what a sweep costs once the memory
+ * pipeline is full, and how far the last workgroup finishes behind the median one.  Only rows
+ * that take the register-ring kernel on 512 threads (385-512 vectors of 16 bytes at a 16-byte
+ * pitch: 4096 bf16/fp16 columns, 2048 fp32 columns) have such a build; other shapes return
+ * MG_ERR_UNSUPPORTED.  records must be zeroed by the caller if unwritten words are to read 0.
+ */
+#define MG_TIMELINE_WORDS 32
+#define MG_TIMELINE_ITERATIONS 24
+int mg_rmsnorm_bwd_timeline(void* dx, float* dw_partial, const void* dy, const void* x, const void* w,
+                            const float* inv_rms, int64_t rows, int64_t cols, int dtype, int64_t num_partials,
+                            int64_t ld, uint64_t* records, void* stream);
+
+/*
  * Tuning hook (not needed for normal use): overrides one launch parameter for the
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
  * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target

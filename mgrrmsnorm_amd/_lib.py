@@ -46,6 +46,7 @@ SIGNATURES = {
     "mg_stream_probe": (_int, [_vp, _vp, _vp, _i64, _vp]),
     "mg_row_probe": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "mg_rmsnorm_launch_info": (_int, [_int, _i64, _int] + [ctypes.POINTER(_int)] * 4),
+    "mg_rmsnorm_bwd_timeline": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _i64, _vp, _vp]),
 }
 
 

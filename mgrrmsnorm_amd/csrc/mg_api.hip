@@ -5,6 +5,7 @@
 #include "megagemm_hip_tuning.h"
 #include "mg_launch.hpp"
 #include "mg_device.hpp"
+#include "rmsnorm_kernels.hpp"
 
 #include <atomic>
 #include <cstdarg>
@@ -358,8 +359,10 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
     return MG_OK;
 }
 
-int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, const void* w, const float* inv_rms,
-                   int64_t rows, int64_t cols, int dtype, int64_t num_partials, int64_t ld, void* stream) {
+// mg_rmsnorm_bwd, and the same launch with per-workgroup time stamps for mg_rmsnorm_bwd_timeline
+static int rmsnorm_bwd_impl(void* dx, float* dw_partial, const void* dy, const void* x, const void* w,
+                            const float* inv_rms, int64_t rows, int64_t cols, int dtype, int64_t num_partials,
+                            int64_t ld, unsigned long long* timeline, void* stream) {
     int rc = check_rmsnorm_dims("mg_rmsnorm_bwd", rows, cols, dtype);
     if (rc != MG_OK) return rc;
     if (num_partials < 1 || num_partials > 65535)
@@ -405,13 +408,33 @@ int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, c
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,
-                       xcd_group_or(0), prefetch < 0 ? bwd_prefetch_default(cfg, row_bytes) : prefetch != 0};
+                       xcd_group_or(0), prefetch < 0 ? bwd_prefetch_default(cfg, row_bytes) : prefetch != 0, timeline};
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },
         [&] { return launch_rmsnorm_bwd<half_t>(cfg, generic, a, s); },
         [&] { return launch_rmsnorm_bwd<bf16_t>(cfg, generic, a, s); });
+    if (e == hipErrorNotSupported && timeline != nullptr)
+        return fail(MG_ERR_UNSUPPORTED, "mg_rmsnorm_bwd_timeline: only rows that take the register-ring kernel on 512 "
+                                        "threads (385-512 16-byte vectors at a 16-byte pitch, e.g. 4096 bf16 columns) "
+                                        "have a time-stamped build");
     if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd: launch", e);
     return MG_OK;
+}
+
+int mg_rmsnorm_bwd(void* dx, float* dw_partial, const void* dy, const void* x, const void* w, const float* inv_rms,
+                   int64_t rows, int64_t cols, int dtype, int64_t num_partials, int64_t ld, void* stream) {
+    return rmsnorm_bwd_impl(dx, dw_partial, dy, x, w, inv_rms, rows, cols, dtype, num_partials, ld, nullptr, stream);
+}
+
+int mg_rmsnorm_bwd_timeline(void* dx, float* dw_partial, const void* dy, const void* x, const void* w,
+                            const float* inv_rms, int64_t rows, int64_t cols, int dtype, int64_t num_partials,
+                            int64_t ld, uint64_t* records, void* stream) {
+    if (records == nullptr || !aligned(records, 8))
+        return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd_timeline: records must be an 8-byte aligned device pointer");
+    if (rows < 1) return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd_timeline: rows must be >= 1");
+    static_assert(MG_TIMELINE_WORDS == kTimelineWords && MG_TIMELINE_ITERATIONS == kTimelineIters, "header and kernel agree");
+    return rmsnorm_bwd_impl(dx, dw_partial, dy, x, w, inv_rms, rows, cols, dtype, num_partials, ld,
+                            reinterpret_cast<unsigned long long*>(records), stream);
 }
 
 int mg_rmsnorm_dw_reduce(float* dw_f32, void* dw_cast, int cast_dtype, const float* dw_partial,

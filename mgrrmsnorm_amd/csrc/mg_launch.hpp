@@ -148,6 +148,7 @@ struct BwdArgs {
     long rows; int cols; int num_partials;
     int xcd_group;
     bool prefetch;  // request row i+1 before reducing row i (costs a second copy of the row in VGPRs)
+    unsigned long long* timeline;  // kFamilyRing with 512 threads per row only: per-workgroup time stamps, or null
 };
 
 // One set of launchers per element type (T = float, _Float16, __bf16), each defined in

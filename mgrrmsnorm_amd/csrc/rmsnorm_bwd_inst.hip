@@ -61,9 +61,19 @@ hipError_t run_lds_sums(const BwdArgs& a, hipStream_t s) {
 template <int TPR, int ITEMS, int DEPTH>
 hipError_t run_ring(const BwdArgs& a, hipStream_t s) {
     constexpr int BLOCK = TPR > 512 ? TPR : 512;
-    return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH>, dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s,
-            (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms,
-        a.rows, a.cols, 1.0f / (float)a.cols);
+    if (a.timeline != nullptr) {
+        // the time-stamped build exists for the 512-thread layout only (the 4096-column shapes)
+        if constexpr (TPR == 512 && ITEMS == 1)
+            return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH, true>,
+                          dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s, (elem_t*)a.dx, a.dw_part, a.ld,
+                          (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows, a.cols,
+                          1.0f / (float)a.cols, a.timeline);
+        else
+            return hipErrorNotSupported;
+    }
+    return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH>, dim3((unsigned)a.num_partials),
+                  dim3(BLOCK), 0, s, (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x,
+                  (const elem_t*)a.w, a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols, (unsigned long long*)nullptr);
 }
 
 template <int TPR, int ITEMS>
@@ -161,6 +171,7 @@ hipError_t by_tpr(int tpr, int items, const BwdArgs& a, hipStream_t s) {
 
 template <>
 hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const BwdArgs& a, hipStream_t s) {
+    if (a.timeline != nullptr && (generic || cfg.family != kFamilyRing)) return hipErrorNotSupported;
     if (generic) {
         hipError_t e = launch(rmsnorm_bwd_dx_generic<elem_t>, dim3((unsigned)a.rows), dim3(256), 0, s,
             (elem_t*)a.dx, (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows,

@@ -821,12 +821,21 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
 // columns: 277-299 against 267), which therefore stay with rmsnorm_bwd_rows.
 // Iterations past the last row of a slot (the loop runs a multiple of DEPTH) work on an empty
 // buffer resource: loads return 0, stores are dropped, the row scale is 0.
+//
+// TRACE = true is the same kernel with time stamps (the 100 MHz constant clock): thread 0 of
+// every workgroup writes a record of kTimelineWords 64-bit words to `timeline` -- [0] start,
+// [1 + i] end of iteration i (the first kTimelineIters of them), [kTimelineWords - 3] end of the
+// row loop, [kTimelineWords - 2] end of the workgroup, [kTimelineWords - 1] the die (XCC) it ran
+// on -- which is what mg_rmsnorm_bwd_timeline returns.  Without TRACE `timeline` is not touched.
 // =================================================================================
-template <typename T, int VEC, int TPR, int ITEMS, int BLOCK, int DEPTH>
+constexpr int kTimelineWords = 32;
+constexpr int kTimelineIters = 24;
+
+template <typename T, int VEC, int TPR, int ITEMS, int BLOCK, int DEPTH, bool TRACE = false>
 __global__ void __launch_bounds__(BLOCK)
 rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                       const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
-                      long rows, int cols, float inv_cols) {
+                      long rows, int cols, float inv_cols, unsigned long long* __restrict__ timeline) {
     static_assert(BLOCK % TPR == 0 && TPR % kWave == 0, "row slots must tile the workgroup");
     static_assert(DEPTH >= 2 && DEPTH <= 4, "2 to 4 register buffers per row slot");
     constexpr int RG = BLOCK / TPR;
@@ -846,6 +855,8 @@ rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, c
     const u32 row_bytes = (u32)cols * (u32)sizeof(T);
 
     __shared__ float red[2][RG][WPR > 1 ? WPR : 1];
+    unsigned long long t_start = 0;
+    if constexpr (TRACE) t_start = wall_clock64();
 
     float acc[ITEMS][EPV];
 #pragma unroll
@@ -925,8 +936,13 @@ rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, c
                 for (int k = 0; k < EPV; ++k) o[k] = __builtin_fmaf(gf[k] * wf[i][k], s, -(xf[k] * c2));
                 buf_store<NW, kStream>(rd, (u32)(lir + i * TPR) * VEC, pack_vec<T, NW>(o));
             }
+            if constexpr (TRACE) {
+                if (tid == 0 && it < kTimelineIters) timeline[wg * kTimelineWords + 1 + it] = wall_clock64();
+            }
         }
     }
+    unsigned long long t_loop = 0;
+    if constexpr (TRACE) t_loop = wall_clock64();
 
     // ---- combine the RG row slots in slot order, write this workgroup's partial row ----
     float* out = dw_part + wg * ld;
@@ -960,6 +976,17 @@ rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, c
         for (int c = tid * 4; c < lim; c += BLOCK * 4) {
             f32x4 v = {dwbuf[c], dwbuf[c + 1], dwbuf[c + 2], dwbuf[c + 3]};
             *reinterpret_cast<f32x4*>(out + c) = v;
+        }
+    }
+    if constexpr (TRACE) {
+        if (tid == 0) {
+            u32 xcc = 0;
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+            unsigned long long* rec = timeline + wg * kTimelineWords;
+            rec[0] = t_start;
+            rec[kTimelineWords - 3] = t_loop;
+            rec[kTimelineWords - 2] = wall_clock64();
+            rec[kTimelineWords - 1] = xcc & 0xfu;
         }
     }
 }

@@ -41,7 +41,8 @@ def test_header_declares_the_expected_entry_points():
         "mg_rmsnorm_dw_reduce", "mg_rmsnorm_bwd_noalloc", "mg_swiglu_fwd", "mg_swiglu_bwd"])
     # measurement and tuning aids live in a header of their own
     assert _declared_in(TUNING_HEADER) == sorted([
-        "mg_set_option", "mg_copy_bytes", "mg_stream_probe", "mg_row_probe", "mg_rmsnorm_launch_info"])
+        "mg_set_option", "mg_copy_bytes", "mg_stream_probe", "mg_row_probe", "mg_rmsnorm_launch_info",
+        "mg_rmsnorm_bwd_timeline"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -145,6 +146,10 @@ def test_copy_bytes_rejects_bad_arguments(lib):
     assert lib.mg_row_probe(FAKE, FAKE, None, -1, 64, 0, None) == -1 and "rows" in _err(lib)
     assert lib.mg_row_probe(None, FAKE, None, 4, 64, 0, None) == -1
     assert lib.mg_row_probe(None, None, None, 0, 64, 0, None) == 0
+    # the time-stamped backward launch: needs a records pointer and at least one row
+    args = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 64, 4096, 2, 256, 4096)
+    assert lib.mg_rmsnorm_bwd_timeline(*args, None, None) == -1 and "records" in _err(lib)
+    assert lib.mg_rmsnorm_bwd_timeline(FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, 4096, 2, 256, 4096, FAKE, None) == -1
 
 
 def _launch_info(lib, backward, cols, dtype):

@@ -37,3 +37,49 @@ def test_row_probe_copies_and_adds(rows, row_bytes, workgroups):
     assert torch.equal(dst[:n], a) and (dst[n:] == 7).all()
     U.check(L.mg_row_probe(dst.data_ptr(), a.data_ptr(), b.data_ptr(), rows, row_bytes, workgroups, U.stream()))
     assert torch.equal(dst[:n], a + b) and (dst[n:] == 7).all()
+
+
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 700, 4000), ("fp32", 300, 2048)])
+def test_backward_timeline_gives_the_same_results_and_sane_time_stamps(dtype, rows, cols):
+    """mg_rmsnorm_bwd_timeline is mg_rmsnorm_bwd with a clock: dx and the partial rows are
+    bit-identical, every workgroup's record is ordered in time and names one of the 8 dies."""
+    L = U.lib()
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=3)
+    xd, dyd, wd = x.cuda(), dy.cuda(), w.cuda()
+    _, s = U.rmsnorm_fwd(xd, wd, 1e-6, dtype)
+    dx_ref, _, _, part_ref = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    P, ld = U.bwd_workspace(rows, cols, dtype)
+    dx = torch.empty_like(xd)
+    part = torch.full((P, ld), float("nan"), dtype=torch.float32, device="cuda")
+    rec = torch.zeros((P, 32), dtype=torch.int64, device="cuda")
+    U.check(L.mg_rmsnorm_bwd_timeline(dx.data_ptr(), part.data_ptr(), dyd.data_ptr(), xd.data_ptr(), wd.data_ptr(),
+                                      s.data_ptr(), rows, cols, U.CODES[dtype], P, ld, rec.data_ptr(), U.stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(dx.view(torch.uint8), dx_ref.view(torch.uint8))
+    assert torch.equal(part.view(torch.int32), part_ref.view(torch.int32))
+    r = rec.cpu()
+    sweeps = -(-rows // P)
+    n = min(sweeps, 24)
+    assert (r[:, 0] > 0).all() and (r[:, 31] >= 0).all() and (r[:, 31] < 8).all()
+    seq = torch.cat([r[:, 0:1], r[:, 1:1 + n], r[:, 29:31]], dim=1)
+    assert (seq[:, 1:] >= seq[:, :-1]).all(), "time stamps of a workgroup are not in order"
+    assert (r[:, 1 + n:25] == 0).all() or sweeps % 4 != 0   # the loop runs a multiple of its depth
+    span_us = (r[:, 30].max() - r[:, 0].min()).item() * 0.01
+    print(f"{dtype} {rows}x{cols}: {P} workgroups, {sweeps} sweeps, first start to last end {span_us:.2f} us")
+    assert 0 < span_us < 5000
+
+
+def test_backward_timeline_refuses_shapes_without_a_time_stamped_build():
+    L = U.lib()
+    rows, cols = 64, 8192     # 1024 threads per row: no such build
+    x, dy, w = U.rmsnorm_inputs(rows, cols, "bf16", seed=3)
+    xd, dyd, wd = x.cuda(), dy.cuda(), w.cuda()
+    _, s = U.rmsnorm_fwd(xd, wd, 1e-6, "bf16")
+    P, ld = U.bwd_workspace(rows, cols, "bf16")
+    dx = torch.empty_like(xd)
+    part = torch.empty((P, ld), dtype=torch.float32, device="cuda")
+    rec = torch.zeros((P, 32), dtype=torch.int64, device="cuda")
+    rc = L.mg_rmsnorm_bwd_timeline(dx.data_ptr(), part.data_ptr(), dyd.data_ptr(), xd.data_ptr(), wd.data_ptr(),
+                                   s.data_ptr(), rows, cols, U.CODES["bf16"], P, ld, rec.data_ptr(), U.stream())
+    assert rc == -2 and "time-stamped build" in L.mg_last_error().decode()
+    torch.cuda.synchronize()
