@@ -90,8 +90,11 @@ int mg_rmsnorm_bwd_timeline(void* dx, float* dw_partial, const void* dy, const v
  * calling process.  Keys: "fwd_tpr", "bwd_tpr" (threads per row: 64...1024, or 8 / 16 / 32 for
  * rows of at most 4 vectors per thread; -1 = never fewer than 64), "fwd_items" (target
  * 16-byte vectors per thread; 0 = automatic), "bwd_block" (1024 or 512 threads per
- * workgroup), "bwd_wg_per_cu", "bwd_partials" (workgroups of the persistent backward grid, which is
- * also the number of partial rows; 0 = automatic), "bwd_prefetch" (1/0: request the next row before reducing
+ * workgroup; 256 = one row slot of 256 threads per workgroup, two workgroups per compute unit,
+ * for rows of up to 512 vectors), "bwd_wg_per_cu", "bwd_partials" (workgroups of the persistent backward grid, which is
+ * also the number of partial rows; 0 = automatic), "bwd_partial_policy" (how the register-ring kernel
+ * on 512 threads per row stores its partial row: 0 default, 1 non-temporal, 2 written through to
+ * memory; other kernels ignore it), "bwd_prefetch" (1/0: request the next row before reducing
  * the current one; -1 = automatic), "narrow_groups" (the row-group layout for rows of at most
  * 64 vectors: 1, 2 or 4 groups in flight, 0 = never, -1 = automatic; a "fwd_tpr" / "fwd_items" /
  * "bwd_tpr" / "bwd_block" override switches the automatic choice off), "bwd_lds" (backward rows

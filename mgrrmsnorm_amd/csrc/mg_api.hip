@@ -31,7 +31,7 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1}, opt_bwd_ring{-1}, opt_bwd_partials{0};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1}, opt_bwd_ring{-1}, opt_bwd_partials{0}, opt_bwd_partial_policy{0};
 
 // Consecutive logical workgroups one die handles at a time in the one-shot streaming
 // kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
@@ -165,6 +165,10 @@ bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
             return true;
         }
     }
+    if (block == 256) {   // one 256-thread row slot per workgroup, on request only
+        const int need = ceil_div(nvec, 256);
+        if (bwd_cfg_ok(esize, 256, need, 256)) { *cfg = {kVec, 256, need, 256}; return true; }
+    }
     if (tpr_ok(tpr)) {
         const int need = round_items(ceil_div(nvec, tpr));
         for (int b : {block, 512, 1024})
@@ -267,7 +271,7 @@ int mg_set_option(const char* key, int value) {
         {"bwd_tpr", &opt_bwd_tpr},
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
-        {"bwd_prefetch", &opt_bwd_prefetch}, {"bwd_ring", &opt_bwd_ring}, {"bwd_partials", &opt_bwd_partials},
+        {"bwd_prefetch", &opt_bwd_prefetch}, {"bwd_ring", &opt_bwd_ring}, {"bwd_partials", &opt_bwd_partials}, {"bwd_partial_policy", &opt_bwd_partial_policy},
     };
     if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
     for (auto& t : table)
@@ -341,6 +345,7 @@ int mg_rmsnorm_bwd_workspace(int64_t rows, int64_t cols, int dtype, int64_t* num
         rg = cfg.block / cfg.tpr;
         dflt_per_cu = cfg.items >= 4 ? 4 : 1;
         if (cfg.block == 1024) dflt_per_cu = 2;   // both fit a compute unit; 5.9 against 5.5-5.8 TB/s with one
+        if (cfg.block == 256) dflt_per_cu = 2;    // as many row slots as the 512-thread workgroups give
         // one vector per lane leaves half the bytes in flight: a second workgroup makes up for it
         if (narrow_tpr(cfg.tpr)) dflt_per_cu = cfg.items == 1 ? 2 : 1;
         if (cfg.family == kFamilyGroups) { rg = (cfg.block / cfg.tpr) * cfg.items; dflt_per_cu = 1; }
@@ -408,7 +413,8 @@ static int rmsnorm_bwd_impl(void* dx, float* dw_partial, const void* dy, const v
     // the persistent grid already walks the rows in order; regrouping its workgroups by die
     // measured within +-2 % either way, so it stays off unless asked for
     const BwdArgs a = {dx, dw_partial, (int)ld, dy, x, w, inv_rms, (long)rows, (int)cols, (int)num_partials,
-                       xcd_group_or(0), prefetch < 0 ? bwd_prefetch_default(cfg, row_bytes) : prefetch != 0, timeline};
+                       xcd_group_or(0), prefetch < 0 ? bwd_prefetch_default(cfg, row_bytes) : prefetch != 0, timeline,
+                       opt_bwd_partial_policy.load()};
     hipError_t e = by_dtype(
         dtype, [&] { return launch_rmsnorm_bwd<float>(cfg, generic, a, s); },
         [&] { return launch_rmsnorm_bwd<half_t>(cfg, generic, a, s); },

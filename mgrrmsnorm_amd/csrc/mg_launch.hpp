@@ -108,7 +108,11 @@ constexpr bool fwd_items_ok(int items) { return items >= 1 && items <= 8 && item
 // thread without spilling, 512-thread workgroups (256 VGPRs) up to 8 (ITEMS in
 // {1,2,3,4,6,8}).  When several row slots share a workgroup their combine buffer
 // (tpr * items * elements-per-vector floats) must fit 64 KiB of LDS.
+// 256-thread workgroups (one row slot of 256 threads, up to 2 vectors each, several workgroups per
+// compute unit) exist on request only ("bwd_block" = 256): they measure slower than two slots in
+// one 512-thread workgroup, and every workgroup adds a partial row.
 constexpr bool bwd_cfg_ok(int esize, int tpr, int items, int block) {
+    if (block == 256) return tpr == 256 && (items == 1 || items == 2);
     return (block == 1024 || block == 512) && tpr <= block &&
            items >= 1 && items <= (block == 1024 ? 2 : kBwdMaxItems) && items != 5 && items != 7 &&
            (tpr == block || tpr * items * (kVec / esize) * 4 <= 65536);
@@ -149,6 +153,8 @@ struct BwdArgs {
     int xcd_group;
     bool prefetch;  // request row i+1 before reducing row i (costs a second copy of the row in VGPRs)
     unsigned long long* timeline;  // kFamilyRing with 512 threads per row only: per-workgroup time stamps, or null
+    int partial_policy;  // kFamilyRing with 512 threads per row only: 0 default stores of the partial row,
+                         // 1 non-temporal, 2 write-through to memory
 };
 
 // One set of launchers per element type (T = float, _Float16, __bf16), each defined in

@@ -71,6 +71,18 @@ hipError_t run_ring(const BwdArgs& a, hipStream_t s) {
         else
             return hipErrorNotSupported;
     }
+    if constexpr (TPR == 512 && ITEMS == 1) {   // the partial row's store policy, on request
+        if (a.partial_policy == 1)
+            return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH, false, kStream>,
+                          dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s, (elem_t*)a.dx, a.dw_part, a.ld,
+                          (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows, a.cols,
+                          1.0f / (float)a.cols, (unsigned long long*)nullptr);
+        if (a.partial_policy == 2)
+            return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH, false, 17>,
+                          dim3((unsigned)a.num_partials), dim3(BLOCK), 0, s, (elem_t*)a.dx, a.dw_part, a.ld,
+                          (const elem_t*)a.dy, (const elem_t*)a.x, (const elem_t*)a.w, a.inv_rms, a.rows, a.cols,
+                          1.0f / (float)a.cols, (unsigned long long*)nullptr);
+    }
     return launch(rmsnorm_bwd_rows_ring<elem_t, kVec, TPR, ITEMS, BLOCK, DEPTH>, dim3((unsigned)a.num_partials),
                   dim3(BLOCK), 0, s, (elem_t*)a.dx, a.dw_part, a.ld, (const elem_t*)a.dy, (const elem_t*)a.x,
                   (const elem_t*)a.w, a.inv_rms, a.rows, a.cols, 1.0f / (float)a.cols, (unsigned long long*)nullptr);
@@ -213,6 +225,7 @@ hipError_t launch_rmsnorm_bwd<elem_t>(const RowCfg& cfg, bool generic, const Bwd
     if (cfg.tpr == 32 && cfg.block == 512) return narrow_by_items<32>(cfg.items, a, s);
     if (cfg.block == 1024) return by_tpr<1024>(cfg.tpr, cfg.items, a, s);
     if (cfg.block == 512) return by_tpr<512>(cfg.tpr, cfg.items, a, s);
+    if (cfg.block == 256 && cfg.tpr == 256) return by_items<256, 256>(cfg.items, a, s);
     return hipErrorInvalidValue;
 }
 

@@ -831,7 +831,7 @@ rmsnorm_bwd_rows(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const 
 constexpr int kTimelineWords = 32;
 constexpr int kTimelineIters = 24;
 
-template <typename T, int VEC, int TPR, int ITEMS, int BLOCK, int DEPTH, bool TRACE = false>
+template <typename T, int VEC, int TPR, int ITEMS, int BLOCK, int DEPTH, bool TRACE = false, int PARTIAL_POLICY = 0>
 __global__ void __launch_bounds__(BLOCK)
 rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, const T* __restrict__ dy,
                       const T* __restrict__ x, const T* __restrict__ w, const float* __restrict__ inv_rms,
@@ -945,16 +945,26 @@ rmsnorm_bwd_rows_ring(T* __restrict__ dx, float* __restrict__ dw_part, int ld, c
     if constexpr (TRACE) t_loop = wall_clock64();
 
     // ---- combine the RG row slots in slot order, write this workgroup's partial row ----
+    // PARTIAL_POLICY (one slot per workgroup only): the cache-policy bits of the partial row's
+    // stores -- 0 default (the row stays in this die's L2 until the end-of-kernel write-back),
+    // kStream non-temporal, 17 (sc0 sc1) written through to memory at once.  Measured at
+    // 4096 x 4096 bf16 they differ by less than the run-to-run spread, so 0 is what runs; the
+    // other two exist for the "bwd_partial_policy" option.
     float* out = dw_part + wg * ld;
     if constexpr (RG == 1) {
+        const rsrc_t rp = make_rsrc(out, (u32)ld * 4u);   // ld < 2^29 floats: cols < 2^31 bytes per row
 #pragma unroll
         for (int i = 0; i < ITEMS; ++i) {
             const int c0 = (lir + i * TPR) * EPV;   // ld % 4 == 0 and EPV % 4 == 0
 #pragma unroll
-            for (int h = 0; h < EPV / 4; ++h)
-                if (c0 + 4 * h < ld)
-                    *reinterpret_cast<f32x4*>(out + c0 + 4 * h) =
-                        f32x4{acc[i][4 * h], acc[i][4 * h + 1], acc[i][4 * h + 2], acc[i][4 * h + 3]};
+            for (int h = 0; h < EPV / 4; ++h) {
+                const f32x4 v = {acc[i][4 * h], acc[i][4 * h + 1], acc[i][4 * h + 2], acc[i][4 * h + 3]};
+                if constexpr (PARTIAL_POLICY == 0) {
+                    if (c0 + 4 * h < ld) *reinterpret_cast<f32x4*>(out + c0 + 4 * h) = v;
+                } else {   // out-of-range offsets are dropped by the buffer's range check
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rp, (c0 + 4 * h) * 4, 0, PARTIAL_POLICY);
+                }
+            }
         }
     } else {
         __shared__ float dwbuf[COVER];

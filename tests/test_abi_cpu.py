@@ -215,6 +215,13 @@ def test_ring_option_switches_the_backward_layout(lib):
     assert _launch_info(lib, 1, 4096, 2) == (0, 512, 1, 512)
     # rows whose pitch is not a multiple of 16 bytes never take the ring
     assert _launch_info(lib, 1, 4100, 2) == (0, 512, 2, 512)
+    # one 256-thread row slot per workgroup exists on request only
+    try:
+        assert lib.mg_set_option(b"bwd_block", 256) == 0
+        assert _launch_info(lib, 1, 4096, 2) == (0, 256, 2, 256)
+        assert _launch_info(lib, 1, 8192, 2) == (0, 1024, 1, 1024) or _launch_info(lib, 1, 8192, 2)[3] != 256
+    finally:
+        assert lib.mg_set_option(b"bwd_block", 0) == 0
 
 
 def test_launch_info_rejects_bad_arguments(lib):
@@ -229,7 +236,7 @@ def test_set_option(lib):
     assert lib.mg_set_option(b"no_such_key", 1) == -1 and "unknown key" in _err(lib)
     assert lib.mg_set_option(None, 1) == -1
     for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_block", b"bwd_wg_per_cu", b"swiglu_unroll",
-                b"force_generic", b"bwd_partials"):
+                b"force_generic", b"bwd_partials", b"bwd_partial_policy"):
         assert lib.mg_set_option(key, 0) == 0
     for key in (b"bwd_ring", b"bwd_lds", b"bwd_prefetch", b"narrow_groups", b"xcd_group"):
         assert lib.mg_set_option(key, -1) == 0

@@ -448,6 +448,59 @@ def test_every_backward_workgroup_shape(block, tpr):
     U.assert_dw(dw, dw_ref)
 
 
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 1000, 4096), ("fp16", 333, 2048), ("bf16", 77, 1000), ("fp32", 500, 2048)])
+def test_one_row_slot_per_workgroup_on_request(dtype, rows, cols):
+    """"bwd_block" = 256: 256-thread workgroups of one row slot each, two per compute unit (an
+    experiment kept reachable through the option; it measures slower than two slots sharing a
+    workgroup).  Same answers; twice the partial rows."""
+    import ctypes
+
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=71)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    L = U.lib()
+    P0, _ = U.bwd_workspace(rows, cols, dtype)
+    U.check(L.mg_set_option(b"bwd_block", 256))
+    try:
+        out = [ctypes.c_int(0) for _ in range(4)]
+        U.check(L.mg_rmsnorm_launch_info(1, cols, U.CODES[dtype], *[ctypes.byref(o) for o in out]))
+        assert (out[1].value, out[3].value) == (256, 256) and out[2].value in (1, 2)
+        P1, _ = U.bwd_workspace(rows, cols, dtype)
+        dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+    finally:
+        U.check(L.mg_set_option(b"bwd_block", 0))
+    assert P1 == min(2 * torch.cuda.get_device_properties(0).multi_processor_count, rows) and P1 >= P0
+    U.assert_matches(dx, dx_ref, dtype, "dx bwd_block=256", floor=floor)
+    U.assert_dw(dw, dw_ref)
+    assert torch.isfinite(part).all()
+
+
+@pytest.mark.parametrize("dtype,rows,cols", [("bf16", 4096, 4096), ("fp16", 300, 3584), ("fp32", 700, 2048)])
+def test_partial_row_store_policies_agree(dtype, rows, cols):
+    """"bwd_partial_policy": default, non-temporal and written-through stores of the partial rows
+    (register-ring kernel on 512 threads) are the same numbers, bit for bit."""
+    x, dy, w = U.rmsnorm_inputs(rows, cols, dtype, seed=72)
+    _, _, dx_ref, dw_ref, floor = U.rmsnorm_reference(x, dy, w, EPS, dtype)
+    xd, dyd, wd = _dev(x, dy, w)
+    _, s = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    L = U.lib()
+    got = []
+    for pol in (0, 1, 2):
+        U.check(L.mg_set_option(b"bwd_partial_policy", pol))
+        try:
+            dx, dw, _, part = U.rmsnorm_bwd(dyd, xd, wd, s, dtype)
+        finally:
+            U.check(L.mg_set_option(b"bwd_partial_policy", 0))
+        assert torch.isfinite(part).all(), f"policy {pol}: padding columns of a partial row were left unwritten"
+        got.append((dx.clone(), part.clone(), dw.clone()))
+    U.assert_matches(got[0][0], dx_ref, dtype, "dx, partial policies", floor=floor)
+    U.assert_dw(got[0][2], dw_ref)
+    for pol in (1, 2):
+        for a, b in zip(got[0], got[pol]):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"policy {pol} differs"
+
+
 @pytest.mark.parametrize("prefetch", [0, 1])
 @pytest.mark.parametrize("cols", [1024, 16384])
 def test_backward_with_and_without_row_prefetch(prefetch, cols):
