@@ -436,8 +436,10 @@ def time_configs(lib):
                 rec["probe_" + kind + "_GB/s"] = round((2 if kind == "copy" else 3) * wl.tensor_bytes / t / 1e9)
             # the same bytes moved by whole rows (a workgroup per row forward, a persistent grid of one
             # workgroup per compute unit backward): what whole-row ownership costs at this row length
+            # (rows of 8 KiB and more: the probe gives every row a workgroup of its own, which shorter
+            # rows do not fill -- the operators put several of those on one workgroup)
             rb = getattr(wl, "row_bytes", 0)
-            if rb and rb % 16 == 0 and rb <= 65536:
+            if rb and rb % 16 == 0 and 8192 <= rb <= 65536:
                 t = time_kernel(wl, None, launches=n_launch, fn=lambda i, st: wl.probe("rows_copy", i, st))
                 rec["probe_rows_copy_GB/s"] = round(2 * wl.tensor_bytes / t / 1e9)
                 if getattr(wl, "backward", False):
