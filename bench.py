@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the RMSNorm / SwiGLU path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--launch graph|eager]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--launch graph|eager|second-stream]
 
 A step is one pass of the hot path over one batch of synthetic input that is already
 resident in HBM.  The default workload is the one the headline metric is quoted on:
@@ -227,14 +227,43 @@ def time_steps(wl, steps, warmup, launch, repeats=5):
             readings.append(time.perf_counter() - t0)
         return sorted(readings)
     st = stream_ptr()
+    step = wl.step
+    if launch == "second-stream":
+        step = second_stream_step(wl)
     for _ in range(repeats):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(steps):
-            wl.step(warmup + i, st)
+            step(warmup + i, st)
         torch.cuda.synchronize()
         readings.append(time.perf_counter() - t0)
     return sorted(readings)
+
+
+def second_stream_step(wl):
+    """A step whose dW reduction goes to a second stream, ordered after backward pass 1 by an
+    event, so that it may overlap the next step's forward pass; the next pass 1 waits for it,
+    since the partial rows are shared.  Same work and results as `wl.step`; measured on request
+    only (`--launch second-stream`): the hand-over between the two queues costs more than the
+    3 us of the reduction it hides."""
+    if not getattr(wl, "backward", False):
+        raise SystemExit("--launch second-stream needs an rmsnorm_fwd_bwd workload")
+    main, side = torch.cuda.current_stream(), torch.cuda.Stream()
+    after_pass1, after_reduce = torch.cuda.Event(), torch.cuda.Event()
+    state = {"reduced": False}
+
+    def step(i, st):
+        wl.fwd(i, st)
+        if state["reduced"]:
+            main.wait_event(after_reduce)
+        wl.bwd_pass1(i, st)
+        after_pass1.record(main)
+        side.wait_event(after_pass1)
+        wl.reduce(i, side.cuda_stream)
+        after_reduce.record(side)
+        state["reduced"] = True
+
+    return step
 
 
 def time_kernel(wl, name, launches=200, fn=None):
@@ -621,8 +650,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="rmsnorm_fwd_bwd_4096x4096_bf16")
-    ap.add_argument("--launch", choices=["graph", "eager", "best"], default="best",
-                    help="how the K timed steps are enqueued: one HIP graph, one by one, or the faster of the two")
+    ap.add_argument("--launch", choices=["graph", "eager", "best", "second-stream"], default="best",
+                    help="how the K timed steps are enqueued: one HIP graph, one by one, or the faster of the two; "
+                         "'second-stream' enqueues them one by one with the dW reduction on a second stream "
+                         "(measured on request only: it is slower)")
     ap.add_argument("--buffer-sets", type=int, default=0,
                     help="input/output buffer sets the steps rotate over; 0 = enough to exceed four times the "
                          "256 MiB Infinity Cache (the reported configuration), 1 = everything stays cache resident")
