@@ -110,6 +110,14 @@ int mg_rmsnorm_bwd_timeline(void* dx, float* dw_partial, const void* dy, const v
  */
 int mg_set_option(const char* key, int value);
 
+/*
+ * Number of successful mg_set_option calls in this process so far.  The answers of
+ * mg_rmsnorm_bwd_workspace and mg_rmsnorm_launch_info depend on the options: a caller that
+ * remembers them (the ctypes binding does) keeps this number beside them and asks again when it
+ * has moved, whoever moved it.
+ */
+int mg_option_generation(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,6 +35,7 @@ SIGNATURES = {
     "mg_abi_version": (_int, []),
     "mg_last_error": (ctypes.c_char_p, []),
     "mg_set_option": (_int, [ctypes.c_char_p, _int]),
+    "mg_option_generation": (_int, []),
     "mg_rmsnorm_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_float, _int, _vp]),
     "mg_rmsnorm_bwd_workspace": (_int, [_i64, _i64, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64)]),
     "mg_rmsnorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _i64, _i64, _vp]),
@@ -128,8 +129,6 @@ class device_of:
 
 
 def set_option(key: str, value: int) -> None:
-    """Tuning hook (mg_set_option); also drops the workspace shapes remembered by ops."""
+    """Tuning hook (mg_set_option).  The workspace shapes the ctypes binding remembers follow
+    the library's own count of option changes, so nothing has to be cleared here."""
     check(load().mg_set_option(key.encode(), int(value)), "mg_set_option")
-    from . import ops_ctypes
-
-    ops_ctypes._workspace_shapes.clear()

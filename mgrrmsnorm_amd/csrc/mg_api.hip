@@ -130,9 +130,10 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
 // Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  From sweeps over
 // 576...16384 columns on MI355X: the fewest threads per row that keep a thread at or below
 // two vectors -- three vectors at half the threads lose 4-23 % (1032 columns: 5.0 against
-// 6.1 TB/s, 4104: 5.4 against 6.1), and one vector at twice the threads loses at the
-// 4096 x 4096 shape (20.5 against 18.9 us).  Rows of more than 1024 vectors take what fits:
-// 512 x 3, 1024 x 2, 512 x 4...8.
+// 6.1 TB/s, 4104: 5.4 against 6.1), and with the copied prefetch one vector at twice the
+// threads loses at the 4096 x 4096 shape (20.5 against 18.9 us; with the ring of register
+// buffers, chosen first below where it applies, it wins).  Rows of more than 1024 vectors take
+// what fits: 512 x 3, 1024 x 2, 512 x 4...8.
 bool choose_bwd(long row_bytes, int esize, RowCfg* cfg) {
     const long nvec = (row_bytes + kVec - 1) / kVec;
     const int tpr = opt_bwd_tpr.load(), block = opt_bwd_block.load();
@@ -264,6 +265,12 @@ int mg_abi_version(void) { return MG_ABI_VERSION; }
 
 const char* mg_last_error(void) { return g_err; }
 
+// Counts the successful mg_set_option calls of this process: whoever remembers an answer that
+// depends on the options (a workspace shape) compares it before trusting the memory.
+static std::atomic<int> g_option_generation{0};
+
+int mg_option_generation(void) { return g_option_generation.load(); }
+
 int mg_set_option(const char* key, int value) {
     if (key == nullptr) return fail(MG_ERR_INVALID_ARG, "mg_set_option: key is NULL");
     struct { const char* k; std::atomic<int>* v; } table[] = {
@@ -273,9 +280,17 @@ int mg_set_option(const char* key, int value) {
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
         {"bwd_prefetch", &opt_bwd_prefetch}, {"bwd_ring", &opt_bwd_ring}, {"bwd_partials", &opt_bwd_partials}, {"bwd_partial_policy", &opt_bwd_partial_policy},
     };
-    if (strcmp(key, "swiglu_max_units") == 0) { set_swiglu_max_units(value); return MG_OK; }
+    if (strcmp(key, "swiglu_max_units") == 0) {
+        set_swiglu_max_units(value);
+        g_option_generation.fetch_add(1);
+        return MG_OK;
+    }
     for (auto& t : table)
-        if (strcmp(t.k, key) == 0) { t.v->store(value); return MG_OK; }
+        if (strcmp(t.k, key) == 0) {
+            t.v->store(value);
+            g_option_generation.fetch_add(1);
+            return MG_OK;
+        }
     return fail(MG_ERR_INVALID_ARG, "mg_set_option: unknown key '%s'", key);
 }
 
@@ -380,7 +395,7 @@ static int rmsnorm_bwd_impl(void* dx, float* dw_partial, const void* dy, const v
         return fail(MG_ERR_INVALID_ARG, "mg_rmsnorm_bwd: dw_partial must be a 16-byte aligned device pointer");
     hipStream_t s = (hipStream_t)stream;
     if (rows == 0) {
-            hipError_t e = launch_fill_zero(dw_partial, (long)(num_partials * ld), s);
+        hipError_t e = launch_fill_zero(dw_partial, (long)(num_partials * ld), s);
         if (e != hipSuccess) return fail_hip("mg_rmsnorm_bwd: zero fill", e);
         return MG_OK;
     }
@@ -397,17 +412,25 @@ static int rmsnorm_bwd_impl(void* dx, float* dw_partial, const void* dy, const v
     if (!generic && cfg.family == kFamilyRing) {
         // Two buffers (one row requested ahead) for rows that fill their lanes, four (three rows
         // ahead) for rows that leave up to a quarter of the lanes idle (bf16, 65536 rows, two / four
-        // buffers / the copying loop: 2048 columns 126.6 / 131.1 / 127.8 us, 4096 columns 261.4 / 273.1 /
-        // 262.0, 768 columns 56.2 / 49.1 / 50.2, 3072 columns 204.5 / 192.2 / 196.2), and four as well
-        // while a slot has at most 32 rows, where filling the memory pipeline at the start counts
-        // (4096 x 4096: 19.2 / 18.8 / 18.9).  Two vectors per thread: always two buffers (registers).
+        // buffers / the copying loop: 2048 columns 125.1 / 128.8 / 127.3 us, 4096 columns 258.4 / 267.6 /
+        // 255.9, 768 columns 56.2 / 48.4 / 49.7, 3072 columns 204.5 / 192.2 / 196.2), and four as well
+        // while a slot has few rows, where filling the memory pipeline at the start counts: up to 32
+        // rows per slot (1024 columns x 32768 rows: 34.4 / 33.1 / 34.0 us), up to 128 with one 512-thread
+        // slot per workgroup (4096 x 4096: 19.0 / 18.45 / 18.8; 16384 x 4096: 66.2 / 63.4 / 64.2; 32768 x
+        // 4096: 129.6 / 128.9 / 127.8; 65536 x 4096 see above).  Rows on 1024 threads keep two: three rows of
+        // 16 KiB requested ahead for x and for dy are more than a compute unit keeps in flight to any
+        // gain (4096 x 8192: 34.5 / 35.1 / 37.2; 16384 x 8192: 125.5 / 126.6 / 129.4).  Two vectors per
+        // thread: always two buffers (registers).
         const int forced = opt_bwd_ring.load();
         const long nvec = (row_bytes + kVec - 1) / kVec;
         const long slots = num_partials * (cfg.block / cfg.tpr);
+        const long rows_per_slot = (rows + slots - 1) / slots;
         const bool full = nvec * 8 > 7L * cfg.tpr;
         if (cfg.items != 1) cfg.depth = 2;
         else if (forced == 2 || forced == 4) cfg.depth = forced;
-        else cfg.depth = (!full || (rows + slots - 1) / slots <= 32) ? 4 : 2;
+        else if (!full) cfg.depth = 4;
+        else if (cfg.tpr >= 1024) cfg.depth = 2;
+        else cfg.depth = rows_per_slot <= (cfg.tpr == 512 ? 128 : 32) ? 4 : 2;
     }
     const int prefetch = opt_bwd_prefetch.load();   // every option is read once per call
     // the persistent grid already walks the rows in order; regrouping its workgroups by die

@@ -73,11 +73,18 @@ def rmsnorm_forward(input: torch.Tensor, weight: torch.Tensor, epsilon: float):
 
 
 # (device index, rows, cols, dtype code) -> (num_partials, ld); the answer depends on nothing else
-# but the tuning options, and _lib.set_option() clears this table (a direct mg_set_option does not)
+# but the tuning options, so the table is dropped whenever the library's count of option changes
+# has moved (through _lib.set_option or a direct mg_set_option alike)
 _workspace_shapes: dict = {}
+_workspace_generation = -1
 
 
 def _bwd_workspace(lib, dev, rows, cols, code):
+    global _workspace_generation
+    generation = lib.mg_option_generation()
+    if generation != _workspace_generation:
+        _workspace_shapes.clear()
+        _workspace_generation = generation
     key = (dev.index, rows, cols, code)
     hit = _workspace_shapes.get(key)
     if hit is None:

@@ -41,8 +41,8 @@ def test_header_declares_the_expected_entry_points():
         "mg_rmsnorm_dw_reduce", "mg_rmsnorm_bwd_noalloc", "mg_swiglu_fwd", "mg_swiglu_bwd"])
     # measurement and tuning aids live in a header of their own
     assert _declared_in(TUNING_HEADER) == sorted([
-        "mg_set_option", "mg_copy_bytes", "mg_stream_probe", "mg_row_probe", "mg_rmsnorm_launch_info",
-        "mg_rmsnorm_bwd_timeline"])
+        "mg_set_option", "mg_option_generation", "mg_copy_bytes", "mg_stream_probe", "mg_row_probe",
+        "mg_rmsnorm_launch_info", "mg_rmsnorm_bwd_timeline"])
 
 
 def test_library_exports_every_declared_symbol(lib):
@@ -240,6 +240,47 @@ def test_set_option(lib):
         assert lib.mg_set_option(key, 0) == 0
     for key in (b"bwd_ring", b"bwd_lds", b"bwd_prefetch", b"narrow_groups", b"xcd_group"):
         assert lib.mg_set_option(key, -1) == 0
+
+
+def test_option_generation_counts_successful_changes_only(lib):
+    g0 = lib.mg_option_generation()
+    assert lib.mg_set_option(b"no_such_key", 1) == -1
+    assert lib.mg_option_generation() == g0
+    assert lib.mg_set_option(b"bwd_tpr", 0) == 0
+    assert lib.mg_set_option(b"swiglu_max_units", 0) == 0
+    assert lib.mg_option_generation() == g0 + 2
+
+
+def test_remembered_workspace_shapes_follow_a_direct_option_change():
+    """The ctypes binding remembers (partial rows, pitch) per shape; an option set by anyone,
+    also not through the package, must make it ask the library again."""
+    import ctypes
+    import types
+
+    from mgrrmsnorm_amd import ops_ctypes
+
+    state = {"generation": 7, "partials": 256, "queries": 0}
+
+    def workspace(rows, cols, code, n_part, ld):
+        state["queries"] += 1
+        ctypes.cast(n_part, ctypes.POINTER(ctypes.c_int64))[0] = state["partials"]
+        ctypes.cast(ld, ctypes.POINTER(ctypes.c_int64))[0] = cols
+        return 0
+
+    fake = types.SimpleNamespace(mg_option_generation=lambda: state["generation"], mg_rmsnorm_bwd_workspace=workspace)
+    dev = types.SimpleNamespace(index=0)
+    saved = (dict(ops_ctypes._workspace_shapes), ops_ctypes._workspace_generation)
+    try:
+        assert ops_ctypes._bwd_workspace(fake, dev, 64, 4096, 2) == (256, 4096)
+        assert ops_ctypes._bwd_workspace(fake, dev, 64, 4096, 2) == (256, 4096)
+        assert state["queries"] == 1
+        state["generation"], state["partials"] = 8, 512      # someone called mg_set_option
+        assert ops_ctypes._bwd_workspace(fake, dev, 64, 4096, 2) == (512, 4096)
+        assert state["queries"] == 2
+    finally:
+        ops_ctypes._workspace_shapes.clear()
+        ops_ctypes._workspace_shapes.update(saved[0])
+        ops_ctypes._workspace_generation = saved[1]
 
 
 def test_fastdiv_matches_integer_division(tmp_path):
