@@ -13,6 +13,10 @@ such readings; all five are in `readings_us_per_step`).
 Buffers rotate over several independent sets whose total size exceeds the 256 MB
 Infinity Cache, so consecutive steps do not find their inputs cached.
 
+Everything runs on the default stream while it is the process's only stream; the HIP-graph
+reading of the default `--launch best` comes last, because capturing a graph creates a stream
+(see --extra-streams for what that changes).
+
 Workloads: rmsnorm_fwd_bwd_4096x4096_bf16 (default), rmsnorm_fwd_4096x4096_fp16,
 rmsnorm_fwd_bwd_16384x8192_bf16, rmsnorm_fwd_bwd_65536x{768,2048,4100,5120,16384}_{bf16,fp16},
 swiglu_fwd_bwd_8192x11008_bf16.
@@ -672,6 +676,10 @@ def main():
                     help="also run backward pass 1 that many times with per-workgroup time stamps "
                          "(mg_rmsnorm_bwd_timeline; shapes of 4096 two-byte columns) and report where a launch spends "
                          "its time ('timeline' in the JSON)")
+    ap.add_argument("--extra-streams", type=int, default=0, metavar="N",
+                    help="create N more HIP streams (one small launch on each) before anything is timed; the timed "
+                         "launches stay on the default stream.  For seeing how the number of streams a process holds "
+                         "changes launches with tens of thousands of workgroups")
     ap.add_argument("--calibrate-copies", type=int, default=0,
                     help="also launch this many plain copies of one activation tensor (mg_copy_bytes), so that a "
                          "counter profile of this run holds a kernel of known HBM traffic, and as many streaming "
@@ -693,6 +701,13 @@ def main():
     wl = make_workload(lib, args.workload, args.buffer_sets)
     log(f"[bench] {wl.name}: {wl.step_bytes / 1e6:.1f} MB algorithmic per step, {wl.nsets} buffer sets, "
         f"device {torch.cuda.get_device_name(0)}")
+    # The default stream has been used by now (the workload's tensors were filled on it), so its
+    # hardware queue is the oldest one; every stream created here adds a newer queue.
+    extra_streams = [torch.cuda.Stream() for _ in range(args.extra_streams)]
+    for s_ in extra_streams:        # kept alive to the end: each holds a hardware queue once used
+        with torch.cuda.stream(s_):
+            torch.zeros(64, device="cuda")
+        torch.cuda.synchronize()
 
     if args.calibrate_copies > 0:
         first = wl.sets[0]
@@ -707,37 +722,41 @@ def main():
         torch.cuda.synchronize()
         log(f"[bench] calibration: {args.calibrate_copies} copies of {nbytes} bytes (traffic 2 x {nbytes} each)")
 
-    modes = ["graph", "eager"] if args.launch == "best" else [args.launch]
+    # "best" measures the steps launched one by one first and as one HIP graph last, after every
+    # other section: capturing a graph makes torch create a stream, and on this machine the number
+    # of streams a process holds changes what launches with tens of thousands of workgroups cost on
+    # the default stream (--extra-streams shows it), so everything else is measured while the
+    # default stream is the only one.
     wall, readings = {}, {}
-    for mode in modes:
-        try:
-            readings[mode] = time_steps(wl, args.steps, args.warmup, mode)
-            wall[mode] = readings[mode][len(readings[mode]) // 2]      # the median reading
-        except RuntimeError as exc:
-            if mode == "graph" and len(modes) > 1:      # "best": the eager measurement still stands
-                log(f"[bench] graph launch not measured: {exc}")
-                torch.cuda.synchronize()
-                continue
-            raise
-        log(f"[bench] {mode}: {wall[mode] / args.steps * 1e6:.2f} us/step")
-    mode = min(wall, key=wall.get)
-    sec_per_step = wall[mode] / args.steps
-    value = wl.step_bytes / sec_per_step / 1e9
 
-    # The headline figures are fixed from here on; everything below adds detail to the same JSON
-    # line, and a failure in one of those sections is recorded under its key instead of losing
-    # the line.
-    out = {
-        "metric": "RMSNorm fwd+bwd HBM GB/s at [4096x4096] bf16" if wl.name == "rmsnorm_fwd_bwd_4096x4096_bf16"
-                  else f"{wl.name} HBM GB/s",
-        "value": round(value, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 6),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
-        "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
-        "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
-        "readings_us_per_step": {m: [round(t / args.steps * 1e6, 3) for t in r] for m, r in readings.items()},
-        "library_source_sha16": library_source_sha16(),
-    }
+    def measure(mode):
+        readings[mode] = time_steps(wl, args.steps, args.warmup, mode)
+        wall[mode] = readings[mode][len(readings[mode]) // 2]      # the median reading
+        log(f"[bench] {mode}: {wall[mode] / args.steps * 1e6:.2f} us/step")
+
+    out = {}
+
+    def headline():
+        mode = min(wall, key=wall.get)
+        sec_per_step = wall[mode] / args.steps
+        value = wl.step_bytes / sec_per_step / 1e9
+        out.update({
+            "metric": "RMSNorm fwd+bwd HBM GB/s at [4096x4096] bf16" if wl.name == "rmsnorm_fwd_bwd_4096x4096_bf16"
+                      else f"{wl.name} HBM GB/s",
+            "value": round(value, 1), "unit": "GB/s", "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
+            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 6),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
+            "config": {"workload": wl.name, **wl.desc, "buffer_sets": wl.nsets, "launch": mode},
+            "launch_modes_us_per_step": {m: round(t / args.steps * 1e6, 3) for m, t in wall.items()},
+            "readings_us_per_step": {m: [round(t / args.steps * 1e6, 3) for t in r] for m, r in readings.items()},
+            "library_source_sha16": library_source_sha16(),
+        })
+
+    measure("eager" if args.launch == "best" else args.launch)
+    # The headline figures stand from here on; everything below adds detail to the same JSON line
+    # (the graph reading of "best" may still replace them if it is the faster one), and a failure
+    # in one of those sections is recorded under its key instead of losing the line.
+    headline()
 
     def section(key, fn):
         try:
@@ -778,15 +797,17 @@ def main():
             log(f"[bench] timeline of backward pass 1: {section('timeline', lambda: timeline(wl, lib, args.timeline))}")
         if not args.no_cpu_baseline:
             log(f"[bench] cpu baseline: {section('cpu_baseline', lambda: cpu_baseline(wl))}")
-        del wl
-        import gc
-
-        gc.collect()
-        torch.cuda.empty_cache()
         if not args.no_configs:
             section("configs", lambda: time_configs(lib))
         if args.sweep:
             section("sweep", lambda: sweep(lib))
+        if args.launch == "best":
+            try:
+                measure("graph")
+                headline()
+            except RuntimeError as exc:      # the eager measurement stands
+                log(f"[bench] graph launch not measured: {exc}")
+                torch.cuda.synchronize()
     finally:
         print(json.dumps(out), flush=True)
 
