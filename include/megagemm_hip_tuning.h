@@ -102,7 +102,10 @@ int mg_rmsnorm_bwd_timeline(void* dx, float* dw_partial, const void* dy, const v
  * vectors on, -1 = automatic), "bwd_ring" (backward rows at 16-byte pitches that fill their
  * lanes at one vector per thread, kept in flight through a ring of register buffers: 0 = never,
  * 2 or 4 = that many buffers, -1 = automatic; a "bwd_tpr" / "bwd_block" override switches it
- * off as well), "swiglu_unroll",
+ * off as well), "fwd_lines" (1 = forward rows of more than 256 vectors whose pitch is a multiple of 8 but not of
+ * 128 bytes take the layout with the 16-byte vectors on the 128-byte lines of the output instead of
+ * counted from the row's first byte, which is faster for some such shapes and slower for others;
+ * 0 = never, the default; a "fwd_tpr" / "fwd_items" override switches it off as well), "swiglu_unroll",
  * "force_generic" (1 = always take the one-element-per-thread kernels, which nothing selects by itself), "xcd_group" (consecutive workgroups
  * handled by one die at a time, 0 = off, -1 = automatic), "swiglu_max_units" (vectors or
  * elements one SwiGLU launch may cover before the input is split by rows; 0 = 2^31).  Returns MG_ERR_INVALID_ARG for

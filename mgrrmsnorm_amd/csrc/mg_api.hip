@@ -31,7 +31,8 @@ int fail_hip(const char* what, hipError_t e) {
 
 // ---- process-wide tuning overrides (0 / -1 = automatic) ----
 std::atomic<int> opt_fwd_tpr{0}, opt_fwd_items{0}, opt_bwd_tpr{0}, opt_bwd_wg_per_cu{0},
-    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1}, opt_bwd_ring{-1}, opt_bwd_partials{0}, opt_bwd_partial_policy{0};
+    opt_swiglu_unroll{0}, opt_force_generic{0}, opt_bwd_block{0}, opt_xcd_group{-1}, opt_bwd_prefetch{-1}, opt_groups{-1}, opt_bwd_lds{-1}, opt_bwd_ring{-1}, opt_bwd_partials{0}, opt_bwd_partial_policy{0},
+    opt_fwd_lines{0};
 
 // Consecutive logical workgroups one die handles at a time in the one-shot streaming
 // kernels (see xcd_remap); the "xcd_group" option overrides it (0 switches the remap off).
@@ -125,6 +126,24 @@ bool choose_fwd(long row_bytes, RowCfg* cfg) {
         }
     }
     return false;
+}
+
+// On request only ("fwd_lines" = 1): forward rows whose pitch is a multiple of 8 but not of 128
+// bytes, with more than 256 vectors and an output whose rows start at multiples of 8 bytes, in
+// the register-resident layout with the vectors on the 128-byte lines of y, so that a wave's
+// store instruction writes whole lines (a "fwd_tpr" / "fwd_items" override switches it off).
+// It is not chosen automatically because it does not win everywhere (bf16, us per launch,
+// this layout against vectors counted from the row's first byte): 65536 x 2052 88.8 / 95.4,
+// 65536 x 2056 88.5 / 93.3, 32768 x 8200 175.9 / 185.2, 65536 x 5000 219.7 / 225.1, 16384 x 20484
+// 228.0 / 232.1, but 65536 x 4100 185.9 / 183.6, 4096 x 4100 14.1 / 13.6, 16384 x 12292 159.1 / 144.5,
+// 16384 x 16380 192.9 / 185.7.
+bool choose_fwd_lines(long row_bytes, bool y_rows_8_aligned, RowCfg* cfg) {
+    if (opt_fwd_lines.load() != 1 || opt_fwd_tpr.load() != 0 || opt_fwd_items.load() != 0 || !y_rows_8_aligned)
+        return false;
+    const LinesShape sh = fwd_lines_shape(row_bytes);
+    if (sh.tpr == 0 || !fwd_lines_ok(row_bytes, sh.tpr, sh.items)) return false;
+    *cfg = {kVec, sh.tpr, sh.items, 0, kFamilyLines};
+    return true;
 }
 
 // Backward: 512-thread workgroups (8 waves, 256 VGPRs per thread).  From sweeps over
@@ -279,6 +298,7 @@ int mg_set_option(const char* key, int value) {
         {"bwd_wg_per_cu", &opt_bwd_wg_per_cu}, {"swiglu_unroll", &opt_swiglu_unroll},
         {"force_generic", &opt_force_generic}, {"bwd_block", &opt_bwd_block}, {"xcd_group", &opt_xcd_group},
         {"bwd_prefetch", &opt_bwd_prefetch}, {"bwd_ring", &opt_bwd_ring}, {"bwd_partials", &opt_bwd_partials}, {"bwd_partial_policy", &opt_bwd_partial_policy},
+        {"fwd_lines", &opt_fwd_lines},
     };
     if (strcmp(key, "swiglu_max_units") == 0) {
         set_swiglu_max_units(value);
@@ -308,7 +328,8 @@ int mg_rmsnorm_fwd(void* y, float* inv_rms, const void* x, const void* w, int64_
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool generic = opt_force_generic.load() != 0;
-    if (!generic) generic = !choose_fwd(row_bytes, &cfg) && !choose_streaming(row_bytes, &cfg);
+    if (!generic && !choose_fwd_lines(row_bytes, aligned(y, 8), &cfg))
+        generic = !choose_fwd(row_bytes, &cfg) && !choose_streaming(row_bytes, &cfg);
     const FwdArgs a = {y, inv_rms, x, w, (long)rows, (int)cols, eps, xcd_group_or(kXcdGroupStreaming)};
     hipStream_t s = (hipStream_t)stream;
     hipError_t e = by_dtype(
@@ -330,8 +351,10 @@ int mg_rmsnorm_launch_info(int backward, int64_t cols, int dtype, int* generic, 
     const long row_bytes = cols * es;
     RowCfg cfg = {0, 0, 0, 0};
     bool gen = opt_force_generic.load() != 0;
-    if (!gen) gen = !(backward ? choose_bwd(row_bytes, es, &cfg) : choose_fwd(row_bytes, &cfg)) &&
-                    !choose_streaming(row_bytes, &cfg);
+    // forward: as for an output at a multiple of 8 bytes, which every allocation is
+    if (!gen && !(backward == 0 && choose_fwd_lines(row_bytes, true, &cfg)))
+        gen = !(backward ? choose_bwd(row_bytes, es, &cfg) : choose_fwd(row_bytes, &cfg)) &&
+              !choose_streaming(row_bytes, &cfg);
     *generic = gen ? 1 : 0;
     *threads_per_row = gen ? 256 : cfg.tpr;
     *vectors_per_thread = gen ? 0 : (cfg.family == kFamilyGroups ? -cfg.items : cfg.items);

@@ -38,7 +38,8 @@ struct RowCfg {
     int family; // kFamilyResident (rows held in registers), kFamilyStreaming (rows read twice) or
                 // kFamilyGroups (narrow rows, one vector per lane; `items` = row groups in flight) or
                 // kFamilyLdsSums (backward: rows in registers, dW sums in LDS) or
-                // kFamilyRing (backward: a ring of `depth` register buffers per row slot)
+                // kFamilyRing (backward: a ring of `depth` register buffers per row slot) or
+                // kFamilyLines (forward: rows in registers, vectors on the 128-byte lines of y)
     int depth;  // kFamilyRing only: register buffers per row slot (2 or 4); 0 = chosen per call
 };
 constexpr int kFamilyResident = 0, kFamilyStreaming = 1;
@@ -61,6 +62,35 @@ constexpr bool bwd_ring_ok(long row_bytes, int tpr, int items, int depth) {
     const bool shape = (items == 1 && (tpr == 64 || tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024)) ||
                        (items == 2 && tpr == 1024);
     return shape && row_bytes % 16 == 0 && nvec <= (long)tpr * items && (depth == 2 || depth == 4);
+}
+// Forward only, on request: the register-resident layout with the vectors on the 128-byte lines of y, for
+// row pitches that are multiples of 8 but not of 128 bytes and rows of more than 256 vectors
+// (4 KiB; measured from there on).
+// The slots of a row start at the line that holds its first byte, so up to 120 bytes of slots
+// lie in front of the row: `fwd_lines_shape` gives the threads per row and vectors per thread
+// for ceil((120 + row bytes) / 16) slots by the rule of the plain layout (the fewest threads at
+// two vectors each; half the threads at three when the second vector would be mostly empty;
+// 512 x 3 for 1025-1536 slots), 0 threads = the row does not take this layout.
+constexpr int kFamilyLines = 5;
+constexpr bool fwd_lines_pitch(long row_bytes) { return row_bytes % 8 == 0 && row_bytes % 128 != 0 && row_bytes > 256 * 16; }
+struct LinesShape { int tpr, items; };
+constexpr LinesShape fwd_lines_shape(long row_bytes) {
+    if (!fwd_lines_pitch(row_bytes)) return {0, 0};
+    const long slots = (row_bytes + 120 + 15) / 16;
+    if (slots > 1024 && slots <= 1536) return {512, 3};
+    for (int t = 128; t <= 1024; t *= 2) {
+        int need = (int)((slots + t - 1) / t);
+        if (need == 7) need = 8;
+        if (need <= 2 || (t == 1024 && need <= 8)) {
+            if (need == 2 && t >= 256 && slots * 10 < (long)t * 12) { t /= 2; need = (int)((slots + t - 1) / t); }
+            return {t, need};
+        }
+    }
+    return {0, 0};
+}
+constexpr bool fwd_lines_ok(long row_bytes, int tpr, int items) {
+    const bool shape = (tpr == 128 || tpr == 256 || tpr == 512 || tpr == 1024) && items >= 1 && items <= 8 && items != 7;
+    return shape && fwd_lines_pitch(row_bytes) && (row_bytes + 120 + 15) / 16 <= (long)tpr * items;
 }
 constexpr bool groups_ok(long row_bytes, int tpr, int groups) {
     const bool lanes = tpr == 1 || tpr == 2 || tpr == 4 || tpr == 8 || tpr == 16 || tpr == 32 || tpr == 64;

@@ -42,6 +42,30 @@ hipError_t by_items(int items, const FwdArgs& a, hipStream_t s) {
     }
 }
 
+template <int TPR, int ITEMS>
+hipError_t run_lines(const FwdArgs& a, hipStream_t s) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    const long grid = (a.rows + RPB - 1) / RPB;
+    return launch(rmsnorm_fwd_rows_lines<elem_t, kVec, TPR, ITEMS>, dim3((unsigned)grid), dim3(BLOCK), 0, s,
+            (elem_t*)a.y, a.inv_rms, (const elem_t*)a.x, (const elem_t*)a.w, a.rows, a.cols, a.eps,
+        1.0f / (float)a.cols, a.xcd_group);
+}
+
+template <int TPR>
+hipError_t lines_by_items(int items, const FwdArgs& a, hipStream_t s) {
+    switch (items) {
+        case 1: return run_lines<TPR, 1>(a, s);
+        case 2: return run_lines<TPR, 2>(a, s);
+        case 3: return run_lines<TPR, 3>(a, s);
+        case 4: return run_lines<TPR, 4>(a, s);
+        case 5: return run_lines<TPR, 5>(a, s);
+        case 6: return run_lines<TPR, 6>(a, s);
+        case 8: return run_lines<TPR, 8>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 template <int TPR, int ITEMS, bool RAGGED>
 hipError_t run_narrow(const FwdArgs& a, hipStream_t s) {
     constexpr int RPB = 256 / TPR;
@@ -132,6 +156,19 @@ hipError_t launch_rmsnorm_fwd<elem_t>(const RowCfg& cfg, bool generic, const Fwd
             case 16: return groups_by_g<16>(cfg.items, a, s);
             case 32: return groups_by_g<32>(cfg.items, a, s);
             default: return groups_by_g<64>(cfg.items, a, s);
+        }
+    }
+    if (cfg.family == kFamilyLines) {
+        // the kernel's own conditions, checked where it is launched: the pitch, enough slots, and an
+        // output whose rows start at multiples of 8 bytes
+        if (!fwd_lines_ok((long)a.cols * (long)sizeof(elem_t), cfg.tpr, cfg.items) ||
+            reinterpret_cast<uintptr_t>(a.y) % 8 != 0)
+            return hipErrorInvalidValue;
+        switch (cfg.tpr) {
+            case 128: return lines_by_items<128>(cfg.items, a, s);
+            case 256: return lines_by_items<256>(cfg.items, a, s);
+            case 512: return lines_by_items<512>(cfg.items, a, s);
+            default: return lines_by_items<1024>(cfg.items, a, s);
         }
     }
     if (cfg.vec == kVec) return by_tpr<kVec>(cfg.tpr, cfg.items, a, s);

@@ -28,6 +28,10 @@
 
 namespace mg {
 
+// A byte offset no buffer resource holds (rows stay below 2^31 bytes): a load there returns 0,
+// a store there is dropped.
+constexpr u32 kOutOfRange = 0xFFFFFFF0u;
+
 // =================================================================================
 // Forward, register-resident.
 //   grid  = ceil(rows / RPB) workgroups, RPB = BLOCK / TPR rows per workgroup
@@ -98,6 +102,115 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
 }
 
 // =================================================================================
+// Forward, register-resident, vectors on the 128-byte lines of y ("lines" layout): for row
+// pitches that are multiples of 8 but not of 128 bytes.  With vector j of a row at the row's
+// first byte + 16 j (the layout above) every store instruction of a wave begins and ends
+// inside a 128-byte line, so every line of y is written in two pieces by two instructions;
+// here slot k of a row covers bytes [16 k, 16 k + 16) counted from the start of the line that
+// holds the row's first byte, i.e. row bytes [16 k - a, 16 k - a + 16) with a = (address of the
+// row in y) mod 128, so a wave's instruction covers whole lines and only the first and last
+// line of a row are shared with its neighbours.  Slots in front of the row get an
+// out-of-range offset (they load 0 and store nothing), the row's end is clipped by the
+// buffer's range check as everywhere.  When a is 8 mod 16 -- every other row of a pitch that
+// is 8 mod 16 -- the row's first 8 bytes are the upper half of slot (a - 8) / 16, which is
+// always a slot of a thread's first vector: that lane moves them with an 8-byte access of
+// its own into and out of the upper two words (the lower two stay 0 and are not stored).
+// x and w are read at the same offsets as y is written, so a thread holds x, w and y of the
+// same columns whatever a is.  Runs on request only: measured on MI355X (bf16, against the
+// layout above) it gains 2-7 % at 2052, 2056, 5000 and 8200 columns and loses 1-10 % at 4100,
+// 12292 and 16380 columns and at 4096 rows (the figures are where the host chooses).
+//   needs: row pitch and the address of y multiples of 8 bytes (a is then a multiple of 8);
+//          TPR * ITEMS >= ceil((120 + row bytes) / 16) slots
+//   grid / block as rmsnorm_fwd_rows
+// =================================================================================
+template <typename T, int VEC, int TPR, int ITEMS>
+__global__ void __launch_bounds__((TPR > 256 ? TPR : 256))
+rmsnorm_fwd_rows_lines(T* __restrict__ y, float* __restrict__ inv_rms, const T* __restrict__ x,
+                       const T* __restrict__ w, long rows, int cols, float eps, float inv_cols, int xcd_group) {
+    static_assert(VEC == 16, "slots are 16 bytes");
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    constexpr int WPR = TPR / kWave;
+    constexpr int NW = VEC / 4;
+    constexpr int EPV = VEC / (int)sizeof(T);
+
+    const int tid = threadIdx.x;
+    const int rg = __builtin_amdgcn_readfirstlane(tid / TPR);
+    const int lir = tid - rg * TPR;
+    const long row = xcd_remap(blockIdx.x, gridDim.x, xcd_group) * RPB + rg;
+    const bool live = row < rows;
+    const u32 row_bytes = (u32)cols * (u32)sizeof(T);
+    const long base = live ? row * (long)cols : 0;
+
+    const rsrc_t rx = make_rsrc(x + base, live ? row_bytes : 0u);
+    const rsrc_t ry = make_rsrc(y + base, live ? row_bytes : 0u);
+    const rsrc_t rw = make_rsrc(w, row_bytes);
+
+    // a row belongs to whole waves, so its skew is uniform over a wave
+    const u32 a = (u32)__builtin_amdgcn_readfirstlane((int)(reinterpret_cast<unsigned long long>(y + base) & 127ull));
+    const bool half = (a & 8u) != 0;
+    const u32 head_off = (half && (u32)lir * (u32)VEC + 8u == a) ? 0u : kOutOfRange;
+    u32 off[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        const u32 slot_byte = (u32)(lir + i * TPR) * (u32)VEC;
+        off[i] = slot_byte >= a ? slot_byte - a : kOutOfRange;
+    }
+
+    Words<NW> xv[ITEMS];
+    Words<NW> wv[ITEMS];
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) xv[i] = buf_load<NW, kStream>(rx, off[i]);
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) wv[i] = buf_load<NW, kKeep>(rw, off[i]);
+    if (half) {   // the lane whose first slot straddles the row's first byte: that slot's own load was out of range
+        const Words<2> hx = buf_load<2, kStream>(rx, head_off);
+        const Words<2> hw = buf_load<2, kKeep>(rw, head_off);
+        xv[0].v[2] |= hx.v[0];
+        xv[0].v[3] |= hx.v[1];
+        wv[0].v[2] |= hw.v[0];
+        wv[0].v[3] |= hw.v[1];
+    }
+
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float f[EPV];
+        unpack_vec<T, NW>(xv[i], f);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) ss = __builtin_fmaf(f[k], f[k], ss);
+    }
+    ss = wave_sum(ss);
+    if constexpr (WPR > 1) {
+        __shared__ float part[RPB][WPR];
+        const int wir = __builtin_amdgcn_readfirstlane(lir / kWave);
+        if ((tid & (kWave - 1)) == 0) part[rg][wir] = ss;
+        __syncthreads();
+        float t = 0.0f;
+#pragma unroll
+        for (int k = 0; k < WPR; ++k) t += part[rg][k];
+        ss = t;
+    }
+    const float s = fast_rsqrt(ss * inv_cols + eps);
+    if (live && lir == 0 && inv_rms != nullptr) inv_rms[row] = s;
+
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+        float xf[EPV], wf[EPV], o[EPV];
+        unpack_vec<T, NW>(xv[i], xf);
+        unpack_vec<T, NW>(wv[i], wf);
+#pragma unroll
+        for (int k = 0; k < EPV; ++k) o[k] = (xf[k] * s) * wf[k];
+        const Words<NW> ov = pack_vec<T, NW>(o);
+        buf_store<NW, kStream>(ry, off[i], ov);
+        if (i == 0 && half) {
+            const Words<2> h = {{ov.v[2], ov.v[3]}};
+            buf_store<2, kStream>(ry, head_off, h);
+        }
+    }
+}
+
+// =================================================================================
 // Narrow rows (at most 4 vectors per lane): TPR = 8, 16 or 32 lanes per row, so a wave
 // carries 64/TPR consecutive rows and a 256-thread workgroup 256/TPR.  One buffer resource
 // spans the wave's rows; lanes past the end of a row, and rows past the end of the matrix,
@@ -106,7 +219,6 @@ rmsnorm_fwd_rows(T* __restrict__ y, float* __restrict__ inv_rms, const T* __rest
 // multiple of 16 bytes: the last vector of a row then reaches into the next row and is
 // trimmed to its own row on load and on store (load_row_vector / store_row_vector).
 // =================================================================================
-constexpr u32 kOutOfRange = 0xFFFFFFF0u;
 
 // Activations of ragged rows take the default cache policy: a row's last vector is stored in
 // pieces, and lines shared by two rows are written by two instructions; the L2 merges those

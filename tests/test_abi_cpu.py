@@ -224,6 +224,36 @@ def test_ring_option_switches_the_backward_layout(lib):
         assert lib.mg_set_option(b"bwd_block", 0) == 0
 
 
+def test_forward_rows_on_the_lines_of_the_output(lib):
+    """"fwd_lines" = 1: pitches that are multiples of 8 but not of 128 bytes, beyond 4 KiB, take a
+    shape that holds the row plus up to 120 bytes of slots in front of it; by default nothing does."""
+    shapes = {          # (cols, dtype) -> (threads per row, vectors per thread)
+        (4100, 2): (256, 3),     # 8200 bytes: 521 slots
+        (5000, 1): (512, 2),     # 10000 bytes: 633 slots
+        (2052, 2): (128, 3),     # 4104 bytes: 265 slots, the second vector of 256 threads would be empty
+        (8200, 2): (512, 3),     # 16400 bytes: 1033 slots
+        (12292, 1): (1024, 2),   # 24584 bytes: 1545 slots
+        (2050, 0): (256, 3),     # fp32 at the pitch of 4100 two-byte columns
+        (16380, 2): (1024, 3),   # 32760 bytes: 2056 slots, eight more than two vectors of 1024 threads hold
+    }
+    others = (4096, 4098, 4102, 2048, 1032, 2040)    # multiples of 128, not of 8, or at most 4 KiB
+    default = {key: _launch_info(lib, 0, key[0], key[1]) for key in list(shapes) + [(c, 2) for c in others]}
+    assert default[(16380, 2)][:3] == (0, 1024, 2)
+    try:
+        assert lib.mg_set_option(b"fwd_lines", 1) == 0
+        for (cols, dtype), (tpr, items) in shapes.items():
+            assert _launch_info(lib, 0, cols, dtype)[:3] == (0, tpr, items), (cols, dtype)
+        for c in others:
+            assert _launch_info(lib, 0, c, 2) == default[(c, 2)], c
+        assert lib.mg_set_option(b"fwd_tpr", 512) == 0       # a forced shape switches the layout off as well
+        assert _launch_info(lib, 0, 4100, 2)[:3] == (0, 512, 2)
+    finally:
+        assert lib.mg_set_option(b"fwd_tpr", 0) == 0
+        assert lib.mg_set_option(b"fwd_lines", 0) == 0
+    for key, shape in default.items():
+        assert _launch_info(lib, 0, key[0], key[1]) == shape, key
+
+
 def test_launch_info_rejects_bad_arguments(lib):
     out = [ctypes.c_int() for _ in range(4)]
     refs = [ctypes.byref(o) for o in out]
@@ -236,7 +266,7 @@ def test_set_option(lib):
     assert lib.mg_set_option(b"no_such_key", 1) == -1 and "unknown key" in _err(lib)
     assert lib.mg_set_option(None, 1) == -1
     for key in (b"fwd_tpr", b"fwd_items", b"bwd_tpr", b"bwd_block", b"bwd_wg_per_cu", b"swiglu_unroll",
-                b"force_generic", b"bwd_partials", b"bwd_partial_policy"):
+                b"force_generic", b"bwd_partials", b"bwd_partial_policy", b"fwd_lines"):
         assert lib.mg_set_option(key, 0) == 0
     for key in (b"bwd_ring", b"bwd_lds", b"bwd_prefetch", b"narrow_groups", b"xcd_group"):
         assert lib.mg_set_option(key, -1) == 0

@@ -144,6 +144,53 @@ def test_generic_kernels_match_oracle(dtype):
     U.assert_dw(dw2, dw_ref)
 
 
+@pytest.mark.parametrize("dtype,rows,cols", [
+    ("bf16", 37, 4100),    # pitch 8200 = 8 mod 16: every other row starts in the middle of a slot
+    ("fp16", 5, 5000),     # pitch 10000 = 16 mod 128: whole slots in front of the row
+    ("bf16", 33, 2052),    # 128 threads x 3 vectors
+    ("bf16", 9, 8200),     # 512 threads x 3 vectors
+    ("fp16", 3, 12292),    # 1024 threads x 2 vectors, pitch 24584 = 8 mod 16
+    ("fp32", 7, 2050),     # fp32 at the same pitch as 4100 two-byte columns
+    ("fp32", 4, 1030),     # the shortest rows that take the layout (4120 bytes)
+    ("bf16", 1, 4100),
+])
+@pytest.mark.parametrize("y_off,x_off", [(0, 0), (8, 8), (40, 0), (120, 16), (16, "element"), (4, 0), ("element", 8)])
+def test_forward_with_the_vectors_on_the_lines_of_the_output(dtype, rows, cols, y_off, x_off):
+    """On request ("fwd_lines" = 1) rows whose pitch is a multiple of 8 but not of 128 bytes put
+    their 16-byte vectors on the 128-byte lines of y.  y and x start `y_off` / `x_off` bytes into 128-byte aligned buffers:
+    every skew of the first row, an x that is skewed differently from y, and outputs at 4 or 2
+    bytes off a multiple of 8, which must fall back to vectors counted from the row's first byte.
+    Bytes around y must stay untouched."""
+    es = torch.empty(0, dtype=U.DTYPES[dtype]).element_size()
+    y_off, x_off = (es if o == "element" else o for o in (y_off, x_off))
+    x, _, w = U.rmsnorm_inputs(rows, cols, dtype, seed=cols + y_off)
+    y_ref, s_ref, _, _, _ = U.rmsnorm_reference(x, x, w, EPS, dtype)
+    xd, wd = _dev(x, w)
+    n, guard = rows * cols, 256 // es
+    td = U.DTYPES[dtype]
+    xbuf = torch.zeros(n + 2 * guard, dtype=td, device="cuda")
+    ybuf = torch.full((n + 2 * guard,), 7.0, dtype=td, device="cuda")
+    assert xbuf.data_ptr() % 128 == 0 and ybuf.data_ptr() % 128 == 0
+    xm = xbuf[guard + x_off // es: guard + x_off // es + n].view(rows, cols)
+    ym = ybuf[guard + y_off // es: guard + y_off // es + n].view(rows, cols)
+    xm.copy_(xd)
+    s = torch.empty(rows, dtype=torch.float32, device="cuda")
+    U.check(U.lib().mg_set_option(b"fwd_lines", 1))
+    try:
+        U.check(U.lib().mg_rmsnorm_fwd(ym.data_ptr(), s.data_ptr(), xm.data_ptr(), wd.data_ptr(), rows, cols, EPS,
+                                       U.CODES[dtype], U.stream()), "mg_rmsnorm_fwd")
+        torch.cuda.synchronize()
+    finally:
+        U.check(U.lib().mg_set_option(b"fwd_lines", 0))
+    U.assert_matches(ym, y_ref, dtype, f"y (lines, y+{y_off}, x+{x_off})")
+    np.testing.assert_allclose(U.as_f32(s), s_ref, rtol=2e-6)
+    lo, hi = guard + y_off // es, guard + y_off // es + n
+    assert bool((ybuf[:lo] == 7.0).all()) and bool((ybuf[hi:] == 7.0).all()), "a store went outside y"
+    # the default layout on the same rows, to the same tolerance
+    y0, _ = U.rmsnorm_fwd(xd, wd, EPS, dtype)
+    U.assert_matches(y0, y_ref, dtype, "y (default layout)")
+
+
 def test_inv_rms_pointer_may_be_null():
     x, _, w = U.rmsnorm_inputs(64, 512, "bf16")
     xd, wd = _dev(x, w)
